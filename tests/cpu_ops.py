@@ -21,8 +21,116 @@ class CpuOps:
         take = token_from[:rows] >= 0
         token_ids[:rows][take] = src[token_from[:rows][take].long()]
 
-    def embed(self, table, token_ids, num_rows):
-        return table[token_ids.long()].to(torch.float32)
+    def embed(self, table, token_ids, num_rows, scale=1.0, positions=None, pos_table=None):
+        x = table[token_ids[:num_rows].long()].to(torch.float32) * scale
+        if pos_table is not None:
+            x = x + pos_table[positions[:num_rows].long()].to(torch.float32)
+        return x
+
+    def softcap(self, logits, cap):
+        return cap * torch.tanh(logits / cap)
+
+    def check_activation(self, name):
+        assert name in ("relu2", "relu", "silu", "gelu_tanh")
+
+    def activation(self, x, name):
+        z = x.to(torch.float32)
+        if name == "relu2":
+            y = torch.relu(z) ** 2
+        elif name == "relu":
+            y = torch.relu(z)
+        elif name == "silu":
+            y = z / (1 + torch.exp(-z))
+        else:
+            y = 0.5 * z * (1 + torch.tanh(0.7978845608028654 * (z + 0.044715 * z ** 3)))
+        return y.to(x.dtype)
+
+    # ---- several residual streams ------------------------------------------------
+    def check_streams(self, streams, width):
+        pass
+
+    def streams_open(self, x, streams):
+        return x[:, None, :].repeat(1, streams, 1).contiguous()
+
+    def streams_norm(self, resid, pending, w_in, weight, eps, out_dtype, rows=None, num_rows=None, shift=None):
+        x = resid
+        if pending is not None:
+            y = self.resolve(pending.y).to(torch.float32)
+            x = torch.einsum("st,rsd->rtd", pending.mix, resid) + pending.out[None, :, None] * y[:, None, :]
+            if rows is None:
+                resid.copy_(x)
+        if rows is not None:
+            x = x[rows[:num_rows].long()]
+        u = torch.einsum("s,rsd->rd", w_in, x)
+        h = weight * u * torch.rsqrt((u * u).mean(dim=-1, keepdim=True) + eps)
+        if shift is None:
+            return h.to(out_dtype)
+        mu, state, step = shift
+        return self.token_shift(h, mu, state, step, out_dtype)
+
+    def token_shift(self, h, mu, state, step, out_dtype):
+        out = torch.empty_like(h)
+        for i in range(step.num_seqs):
+            r0, r1 = step.h_row_start[i], step.h_row_start[i + 1]
+            slot = step.h_slots[i]
+            first = state[slot].clone() if step.h_seq_start[i] > 0 else torch.zeros_like(state[slot])
+            prev = torch.cat([first[None], h[r0:r1 - 1]], dim=0)
+            out[r0:r1] = h[r0:r1] + (prev - h[r0:r1]) * mu
+            state[slot] = h[r1 - 1]
+        return out.to(out_dtype)
+
+    # ---- attention with convolved queries and keys, values = keys ----------------------
+    def check_conv_attention_sizes(self, heads, kv_heads, head_dim, taps):
+        pass
+
+    def conv_key_attention(self, qk, bias, conv, state, step, cache, heads, kv_heads, head_dim, taps, scale,
+                           temp, penalty, mask):
+        T = step.num_rows
+        qd = heads * head_dim
+        raw = qk.to(torch.float32)
+        mixed = torch.empty_like(raw)
+        for i in range(step.num_seqs):
+            r0, r1 = step.h_row_start[i], step.h_row_start[i + 1]
+            slot, start = step.h_slots[i], step.h_seq_start[i]
+            if taps > 1:
+                before = state[slot].to(torch.float32).clone()
+                known = torch.arange(start - taps + 1, start) >= 0          # positions before 0 hold nothing
+                hist = torch.where(known[:, None], before + bias, torch.zeros_like(before))
+                u = torch.cat([hist, raw[r0:r1] + bias], dim=0)
+                state[slot] = torch.cat([before, raw[r0:r1]], dim=0)[-(taps - 1):].to(state.dtype)
+            else:
+                u = raw[r0:r1] + bias
+            n = r1 - r0
+            mixed[r0:r1] = sum(conv[:, j] * u[j:j + n] for j in range(taps))
+        q = mixed[:, :qd].to(qk.dtype).to(torch.float32).reshape(T, heads, head_dim)
+        k = mixed[:, qd:].reshape(T, kv_heads, head_dim)
+        page = cache.group.page_size
+        tables = cache.group.tables
+        pos = step.positions[:T].long()
+        seq = step.seq_of_row[:T].long()
+        pages = tables[seq, pos // page].long()
+        assert (pages >= 0).all(), "a row writes to a page that is not held"
+        cache.record("k")[pages, :, pos % page] = k.to(cache.record("k").dtype)
+        out = torch.zeros(T, heads, head_dim)
+        mul = heads // kv_heads
+        for r in range(T):
+            p = int(pos[r])
+            lo = 0
+            if mask is not None:
+                lo = p // mask[1] * mask[1] if mask[0] == "chunk" else max(0, p - mask[1] + 1)
+            idx = torch.arange(lo, p + 1)
+            pg = tables[int(seq[r]), idx // page].long()
+            assert (pg >= 0).all(), "a row reads a page that is not held"
+            kk = cache.record("k")[pg, :, idx % page].to(torch.float32)          # [n, kv, d]
+            dist = (p - idx).to(torch.float32)
+            for h in range(heads):
+                s = (kk[:, h // mul] @ q[r, h]) * scale
+                if temp is not None:
+                    s = s * temp[h]
+                if penalty is not None:
+                    s = s - penalty[0][h] * torch.log(1.0 + penalty[1][h] * dist)
+                out[r, h] = torch.softmax(s, dim=0) @ kk[:, h // mul]
+        return out.reshape(T, qd).to(qk.dtype)
 
     def add_rmsnorm(self, resid, delta, weight, eps, out_dtype, rows=None, num_rows=None, lazy=False):
         if rows is None:

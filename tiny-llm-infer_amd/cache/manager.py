@@ -76,15 +76,39 @@ class CacheRecord:
 class CacheNeed:
     """What one mixer needs of the paged cache: the records it keeps for every token and
     how far back its rows read (``window`` None: everything, else the last ``window``
-    tokens, so that pages before the window can be given back).  Cache layers whose needs
-    are equal share a group: page ids, block tables and tensors of their own."""
+    tokens, so that pages before the window can be given back; ``chunk``: only the positions
+    of its own block of that many, so that the pages of blocks that have passed can).  Cache
+    layers whose needs are equal share a group: page ids, block tables and tensors of their own."""
     records: Tuple[CacheRecord, ...]
     window: Optional[int] = None
+    chunk: Optional[int] = None          # rows read only inside their own block of ``chunk`` positions (counted from 0)
 
     def __post_init__(self):
         names = [r.name for r in self.records]
         if not names or len(set(names)) != len(names):
             raise ValueError("a cache need names at least one record, each once")
+        if self.window is not None and self.chunk is not None:
+            raise ValueError("a cache need has a window or a chunk, not both")
+        if (self.window is not None and self.window <= 0) or (self.chunk is not None and self.chunk <= 0):
+            raise ValueError("a window or a chunk must be positive")
+
+    @property
+    def keeps_all(self) -> bool:
+        """No page of a live request can ever be given back before the request ends."""
+        return self.window is None and self.chunk is None
+
+    @property
+    def reach(self) -> Optional[int]:
+        """A row reads fewer than this many positions back (None: any number)."""
+        return self.window if self.window is not None else self.chunk
+
+    def first_read(self, position: int) -> int:
+        """The lowest position that a row at ``position``, or any later row, reads."""
+        if self.window is not None:
+            return max(0, position - self.window + 1)
+        if self.chunk is not None:
+            return position // self.chunk * self.chunk
+        return 0
 
     @staticmethod
     def keys_and_values(num_kv_heads: int, head_dim: int, window: Optional[int] = None) -> "CacheNeed":
@@ -97,7 +121,9 @@ class CacheNeed:
 
 @dataclass(frozen=True)
 class StateNeed:
-    """Fixed-size state per request: ``shape`` elements of ``dtype`` (a torch dtype)."""
+    """Fixed-size state per request: ``shape`` elements of ``dtype`` (a torch dtype; None: the
+    run's storage type).  A slot is not cleared when it changes hands: whoever keeps state in
+    it treats a sequence that starts at position 0 as having none."""
     shape: Tuple[int, ...]
     dtype: object
 
@@ -199,8 +225,8 @@ class CacheManager:
             raise ValueError("page_size, num_pages and max_requests must be positive")
         distinct = group_needs(needs)
         if per_group is None:
-            per_group = [num_pages if (n.window is None or max_step_tokens is None) else
-                         min(num_pages, window_group_pages(n.window, page_size, max_requests, max_step_tokens))
+            per_group = [num_pages if (n.keeps_all or max_step_tokens is None) else
+                         min(num_pages, window_group_pages(n.reach, page_size, max_requests, max_step_tokens))
                          for n in distinct]
         if len(per_group) != len(distinct):
             raise ValueError(f"{len(per_group)} page counts for {len(distinct)} groups of cache layers")
@@ -220,12 +246,12 @@ class CacheManager:
                 self.groups.append(g)
             g.cache_layers.append(layer)
             self.group_of_layer[layer] = g.index
-        self._no_window = all(g.need.window is None for g in self.groups)
+        self._no_window = all(g.need.keeps_all for g in self.groups)
         self._free_slots = list(range(max_requests - 1, -1, -1))   # pop() gives the lowest
         self._live: Dict[Hashable, RequestCache] = {}
         self.pages_taken_total = 0
         self.pages_returned_total = 0
-        if prefix_caching and any(g.need.window is not None for g in self.groups):
+        if prefix_caching and any(not g.need.keeps_all for g in self.groups):
             raise ValueError("prefix caching needs every layer to keep all keys (no window)")
         self.prefix_caching = prefix_caching
         # per group: hash -> page, and per page its (hash, token ids) while it is in the cache
@@ -342,9 +368,7 @@ class CacheManager:
     # ---- pages ----------------------------------------------------------
     def _first_needed_block(self, g: GroupLayout, first_query_pos: int) -> int:
         """Lowest block a query at ``first_query_pos`` (and any later one) can read."""
-        if g.need.window is None:
-            return 0
-        return max(0, first_query_pos - g.need.window + 1) // self.page_size
+        return g.need.first_read(first_query_pos) // self.page_size
 
     def pages_needed(self, key: Hashable, new_total: int) -> List[int]:
         """Per group, pages that must be taken so that the request can run the
@@ -373,10 +397,10 @@ class CacheManager:
         whole = _blocks(total_tokens, self.page_size)
         out = []
         for g in self.groups:
-            if g.need.window is None:
+            if g.need.keeps_all:
                 out.append(whole)
             else:
-                out.append(min(whole, _blocks(g.need.window - 1, self.page_size) + 2
+                out.append(min(whole, _blocks(g.need.reach - 1, self.page_size) + 2
                                + _blocks(min(portion, total_tokens), self.page_size)))
         return out
 
@@ -385,7 +409,7 @@ class CacheManager:
 
     def _ahead_needed(self, rc: RequestCache, total: int) -> List[int]:
         nb = _blocks(total, self.page_size)
-        return [max(0, nb - len(rc.tables[gi])) if g.need.window is None else 0
+        return [max(0, nb - len(rc.tables[gi])) if g.need.keeps_all else 0
                 for gi, g in enumerate(self.groups)]
 
     def can_hold_ahead(self, key: Hashable, total: int) -> bool:
@@ -403,7 +427,7 @@ class CacheManager:
             raise CacheFull(f"not enough free pages to hold {total} tokens of {key!r}")
         nb = _blocks(total, self.page_size)
         for gi, g in enumerate(self.groups):
-            if g.need.window is None:
+            if g.need.keeps_all:
                 table = rc.tables[gi]
                 while len(table) < nb:
                     table.append(self._take(gi))
@@ -442,7 +466,7 @@ class CacheManager:
                              f"{rc.reserved_tokens} were reserved")
         rc.num_tokens = new_total
         for gi, g in enumerate(self.groups):
-            if g.need.window is None:
+            if g.need.keeps_all:
                 continue
             table = rc.tables[gi]
             first = min(self._first_needed_block(g, new_total), len(table))

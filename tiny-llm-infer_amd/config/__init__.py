@@ -1,6 +1,7 @@
 from .base import (BlockSpec, ConfigError, JsonReader, LayerCall, ModelSpec, PartSpec,
                    read_config_json)
 from .qwen3 import Qwen3Config
+from .sinepel import SinepelConfig
 
 __all__ = ["BlockSpec", "ConfigError", "JsonReader", "LayerCall", "ModelSpec", "PartSpec",
-           "read_config_json", "Qwen3Config"]
+           "read_config_json", "Qwen3Config", "SinepelConfig"]

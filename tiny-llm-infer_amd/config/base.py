@@ -41,6 +41,11 @@ class BlockSpec:
     mixer: PartSpec
     ffn: Optional[PartSpec]
     norms: Dict[str, PartSpec]
+    # what the arrangement itself has beyond its parts: constants, weights of its own by role,
+    # and further parts by role (a token shift in front of the mixer)
+    params: Dict[str, Any] = field(default_factory=dict)
+    names: Dict[str, str] = field(default_factory=dict)
+    parts: Dict[str, PartSpec] = field(default_factory=dict)
 
 
 @dataclass(frozen=True)

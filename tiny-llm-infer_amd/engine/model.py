@@ -21,11 +21,15 @@ class Model:
             mixer = build_part("mixer", b.mixer)
             ffn = build_part("ffn", b.ffn) if b.ffn is not None else None
             norms = {role: build_part("norm", s) for role, s in b.norms.items()}
-            self.blocks.append(build_part("block", PartSpec(b.arrangement), mixer, ffn, norms))
+            self.blocks.append(build_part("block", PartSpec(b.arrangement, dict(b.params), dict(b.names), dict(b.parts)),
+                                          mixer, ffn, norms))
         self.final_norm = build_part("norm", spec.final_norm)
         self.head = build_part("head", spec.head)
         self.schedule = list(spec.schedule)
         self._check_schedule()
+        streams = {b.streams for b in self.blocks}
+        if len(streams) > 1:
+            raise ConfigError(f"the blocks of one model keep the residual in {sorted(streams)} streams; they must agree")
 
     def _check_schedule(self) -> None:
         written = set()
@@ -56,8 +60,21 @@ class Model:
         return [self._needs.get(i) for i in range(self.spec.num_cache_layers())]
 
     def state_needs(self) -> List[Optional[StateNeed]]:
-        """Per run-order entry: the fixed-size state its mixer keeps per request."""
-        return [self.blocks[c.block].mixer.state_need() for c in self.schedule]
+        """Per run-order entry: the fixed-size state its block keeps per request (one need, or
+        several by name)."""
+        return [self.blocks[c.block].state_need() for c in self.schedule]
+
+    def open_residual(self, x: torch.Tensor) -> torch.Tensor:
+        """The residual as the blocks keep it, from the embedding's rows."""
+        return self.blocks[self.schedule[0].block].open(x) if self.schedule else x
+
+    def close_residual(self, resid, pending, rows=None, num_rows=None):
+        """The final norm's rows (of ``rows`` only, if given) from the residual and what the last
+        block still owes it."""
+        if not self.schedule:
+            from ..parts.base import run_norm
+            return run_norm(self.final_norm, resid, pending, rows=rows, num_rows=num_rows)
+        return self.blocks[self.schedule[-1].block].close(resid, pending, self.final_norm, rows, num_rows)
 
     def tensors(self) -> List[TensorDecl]:
         out = self.embedding.tensors()

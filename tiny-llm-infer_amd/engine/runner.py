@@ -128,10 +128,12 @@ class ModelRunner:
                                       dtype=rec.dtype or env.dtype, device=env.device)
                 for rec in g.need.records})
         self.pad_pages, self.pad_slot = [g.pool.num_pages for g in self.cache.groups], max_requests
-        self.states: List[Optional[torch.Tensor]] = []
+        def slots_of(need):
+            return torch.zeros((max_requests + 1,) + tuple(need.shape), dtype=need.dtype or env.dtype, device=env.device)
+        self.states: List = []               # per run-order entry: None, a tensor, or tensors by name
         for need in model.state_needs():
-            self.states.append(None if need is None else torch.zeros(
-                (max_requests + 1,) + tuple(need.shape), dtype=need.dtype, device=env.device))
+            self.states.append(None if need is None else
+                               {k: slots_of(n) for k, n in need.items()} if isinstance(need, dict) else slots_of(need))
         max_width = _pow2_at_least((self.max_model_len + page_size - 1) // page_size)
         self.inputs = StepInputs(env.device, max(max_batch_tokens, _decode_bucket(max_requests)),
                                  _decode_bucket(max_requests), len(self.cache.groups), max_width)
@@ -288,7 +290,7 @@ class ModelRunner:
 
     def _forward(self, step: StepView, num_wanted: int) -> Optional[torch.Tensor]:
         model = self.model
-        resid = model.embedding.forward(step.token_ids, step.num_rows)
+        resid = model.open_residual(model.embedding.forward(step.token_ids, step.num_rows, step.positions))
         pending = None
         for i, call in enumerate(model.schedule):
             if call.cache >= 0 and call.cache in self.cache.group_of_layer:
@@ -304,7 +306,7 @@ class ModelRunner:
         step.state = None
         if num_wanted == 0:
             return None
-        x = run_norm(model.final_norm, resid, pending, rows=step.sample_rows, num_rows=num_wanted)
+        x = model.close_residual(resid, pending, rows=step.sample_rows, num_rows=num_wanted)
         return model.head.forward(x)
 
     def _replay(self, view: StepView, wanted: int) -> torch.Tensor:

@@ -18,7 +18,7 @@ def page_bytes(model, page_size: int, windowed=None) -> int:
     those that keep all keys, True those with a window): every record that the mixers declared."""
     total = 0
     for need in model.cache_needs():
-        if need is not None and (windowed is None or (need.window is not None) == windowed):
+        if need is not None and (windowed is None or (not need.keeps_all) == windowed):
             total += need_page_bytes(need, page_size, model.env.dtype)
     return total
 
@@ -33,8 +33,8 @@ def window_bytes(model, page_size: int, max_batch_tokens: int, max_num_seqs: int
     from ..cache.manager import window_group_pages
     total = 0
     for need in model.cache_needs():
-        if need is not None and need.window is not None:
-            pages = window_group_pages(need.window, page_size, max_num_seqs, max_batch_tokens)
+        if need is not None and not need.keeps_all:
+            pages = window_group_pages(need.reach, page_size, max_num_seqs, max_batch_tokens)
             total += pages * need_page_bytes(need, page_size, model.env.dtype)
     return total
 

@@ -1,7 +1,7 @@
 """Interfaces of the parts a model is put together from, and their registries.
 
 Kinds of parts: position encoding, norm, mixer, feed-forward, block
-(arrangement), embedding, head.  A part is built from a ``PartSpec`` alone: its
+(arrangement), embedding, head, shift (a mix of each row with the row before it).  A part is built from a ``PartSpec`` alone: its
 sizes and constants are ``spec.params``, the checkpoint names of its weights
 are ``spec.names``, nested parts are ``spec.parts``.  Life cycle:
 
@@ -85,7 +85,7 @@ class StepView:
     groups: List[GroupView] = field(default_factory=list)
     # filled by the runner for the layer call that is running
     cache: Optional[LayerCache] = None
-    state: Optional[torch.Tensor] = None      # [slots, *StateNeed.shape] of the running mixer
+    state: Any = None             # of the running block: [slots, *StateNeed.shape], or such tensors by name
 
 
 class Part:
@@ -205,14 +205,28 @@ class Block(Part):
     still owes the residual (None for the first); returns the new pending."""
     mixer: Mixer
     ffn: FeedForward
+    streams = 1          # copies of the residual stream that the arrangement keeps side by side
 
     def forward(self, resid: torch.Tensor, pending: Optional[torch.Tensor],
                 step: StepView) -> torch.Tensor:
         raise NotImplementedError
 
+    def state_need(self):
+        """What the block keeps per request besides the cache: its mixer's need, or a dict of
+        needs by name when several of its parts keep something."""
+        return self.mixer.state_need()
+
+    def open(self, x: torch.Tensor) -> torch.Tensor:
+        """The residual as this arrangement keeps it, from the embedding's rows (float32 [T, n])."""
+        return x
+
+    def close(self, resid, pending, final_norm: "Norm", rows=None, num_rows=None):
+        """The final norm's rows from the residual and what the last block still owes it."""
+        return run_norm(final_norm, resid, pending, rows=rows, num_rows=num_rows)
+
 
 _REGISTRIES: Dict[str, Dict[str, Callable[[PartSpec], Part]]] = {
-    "position": {}, "norm": {}, "mixer": {}, "ffn": {}, "block": {}, "embedding": {}, "head": {},
+    "position": {}, "norm": {}, "mixer": {}, "ffn": {}, "block": {}, "embedding": {}, "head": {}, "shift": {},
 }
 
 

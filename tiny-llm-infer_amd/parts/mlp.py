@@ -1,7 +1,8 @@
 """Dense gated feed-forward: down( silu(gate(x)) * up(x) ) with
 silu(g) = g / (1 + exp(-g)) (model/src/qwen3_paged_batch.cpp:281-295,
 kernels/src/swiglu_kernel_cpu.cpp:20-24).  gate and up are stacked into one
-matrix so that one product reads x once."""
+matrix so that one product reads x once.  And the dense feed-forward without a gate,
+down( act(up(x)) ), for a named activation."""
 from __future__ import annotations
 
 from typing import Dict, List
@@ -45,4 +46,36 @@ class SwiGLU(FeedForward):
         return ops.linear(ops.linear_swiglu(x, self.w_gate_up), self.w_down, deferred=True)   # a delta for the next norm
 
 
+class DenseFF(FeedForward):
+    """Dense feed-forward without a gate: down( act(up(x)) ).  ``activation`` names the
+    function, one of the kernel library's ``ACTIVATIONS`` ("relu2" is relu(z)^2)."""
+    replayable = True
+
+    def __init__(self, spec):
+        super().__init__(spec)
+        self.hidden = int(spec.params["hidden_size"])
+        self.inter = int(spec.params["intermediate_size"])
+        self.activation = str(spec.params["activation"])
+
+    def tensors(self) -> List[TensorDecl]:
+        n = self.spec.names
+        return [TensorDecl(n["up"], (self.inter, self.hidden)),
+                TensorDecl(n["down"], (self.hidden, self.inter))]
+
+    def load(self, weights: Dict[str, torch.Tensor], env: BuildEnv) -> None:
+        super().load(weights, env)
+        n = self.spec.names
+        env.ops.check_activation(self.activation)
+        self.w_up = as_matrix(weights[n["up"]], env)
+        self.w_down = as_matrix(weights[n["down"]], env)
+
+    def workspace_elems(self, rows: int) -> int:
+        return rows * 2 * self.inter
+
+    def forward(self, x: torch.Tensor, step: StepView) -> torch.Tensor:
+        ops = self.env.ops
+        return ops.linear(ops.activation(ops.linear(x, self.w_up), self.activation), self.w_down, deferred=True)
+
+
 register_part("ffn", "swiglu", SwiGLU)
+register_part("ffn", "dense_act", DenseFF)

@@ -1,5 +1,5 @@
 """The one registry from an architecture's name (``architectures[0]`` of its
-config.json) to what builds it: a typed configuration reader and a function
+config.json, or its ``architecture``) to what builds it: a typed configuration reader and a function
 that turns that configuration into an architecture-neutral ``ModelSpec``.
 
 The reference has no registry; it constructs its one model class directly
@@ -42,8 +42,11 @@ def lookup_architecture(name: str) -> Architecture:
 
 def architecture_of(config_json: Dict[str, Any], origin: str = "config.json") -> Architecture:
     archs = config_json.get("architectures")
+    if archs is None and isinstance(config_json.get("architecture"), str):
+        return lookup_architecture(config_json["architecture"])      # one name under the singular key
     if not isinstance(archs, list) or not archs or not isinstance(archs[0], str):
-        raise ConfigError(f"{origin}: 'architectures' must be a non-empty list of names")
+        raise ConfigError(f"{origin}: 'architectures' must be a non-empty list of names "
+                          f"(or 'architecture' one name)")
     return lookup_architecture(archs[0])
 
 

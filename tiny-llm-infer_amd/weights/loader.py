@@ -28,7 +28,8 @@ from .safetensors_io import Checkpoint, write_safetensors
 class TensorDecl:
     name: str
     shape: Tuple[int, ...]
-    init: str = "normal"      # "normal": N(0, 0.02); "ones_normal": 1 + N(0, 0.02); "int": zeros
+    init: str = "normal"      # "normal": N(0, 0.02); "ones_normal": 1 + N(0, 0.02); "int": zeros;
+                              # "normal(m,s)": N(m, s); "abs_normal(m,s)": |N(m, s)|
 
 
 class WeightError(ValueError):
@@ -124,11 +125,20 @@ def random_tensor(decl: TensorDecl, seed: int, index: int, dtype: torch.dtype,
     the same bits wherever it is drawn (``random_init.draw_normal``), then rounded to ``dtype``."""
     if decl.init == "int":
         return torch.zeros(decl.shape, dtype=torch.int32, device=device)
-    if decl.init not in ("normal", "ones_normal"):
-        raise ValueError(f"unknown initialisation '{decl.init}' for {decl.name}")
     from .random_init import draw_normal
-    t = draw_normal(tuple(decl.shape), seed, index, std, 1.0 if decl.init == "ones_normal" else 0.0, device)
-    return t.to(dtype)
+    kind, mean = decl.init, 0.0
+    if "(" in kind:                               # "normal(m,s)", "abs_normal(m,s)"
+        try:
+            kind, args = kind[:-1].split("(")
+            mean, std = (float(a) for a in args.split(","))
+        except ValueError:
+            raise ValueError(f"unknown initialisation '{decl.init}' for {decl.name}") from None
+    elif kind == "ones_normal":
+        kind, mean = "normal", 1.0
+    if kind not in ("normal", "abs_normal"):
+        raise ValueError(f"unknown initialisation '{decl.init}' for {decl.name}")
+    t = draw_normal(tuple(decl.shape), seed, index, std, mean, device)
+    return (t.abs() if kind == "abs_normal" else t).to(dtype)
 
 
 def random_tensors(decls: Sequence[TensorDecl], seed: int, dtype: torch.dtype,
