@@ -293,3 +293,104 @@ extern "C" int tli_swiglu(const void* gu, void* out, int rows, int inter, int dt
         return tli_fail("swiglu: unknown dtype %d", dtype);
     return tli_check_launch("swiglu");
 }
+
+// embed with a scale and learned positions: out[t, :] = scale * E[id[t], :] + P[position[t], :], in float32
+// (P may be absent).  One workgroup a row.
+template <typename T>
+__global__ void embed_scaled_kernel(const T* __restrict__ table, const int* __restrict__ ids,
+                                    const T* __restrict__ pos_table, const int* __restrict__ positions,
+                                    float* __restrict__ out, int hidden, int vocab, int npos, float scale) {
+    const int row = blockIdx.x;
+    int id = ids[row];
+    if (id < 0 || id >= vocab) id = 0;          // the host rejects such ids before the launch
+    const T* src = table + (size_t)id * hidden;
+    const T* pv = nullptr;
+    if (pos_table) {
+        int p = positions[row];
+        if (p < 0 || p >= npos) p = 0;          // the host checks the longest sequence against the table
+        pv = pos_table + (size_t)p * hidden;
+    }
+    float* dst = out + (size_t)row * hidden;
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+        const float e = scale * to_f32(src[i]);
+        dst[i] = pv ? e + to_f32(pv[i]) : e;
+    }
+}
+
+extern "C" int tli_embed_scaled(const void* table, const int* ids, const void* pos_table, const int* positions,
+                                float* out, int rows, int hidden, int vocab, int npos, float scale, int dtype,
+                                void* stream) {
+    if (rows <= 0) return 0;
+    if (hidden <= 0 || vocab <= 0) return tli_fail("embed: bad sizes hidden=%d vocab=%d", hidden, vocab);
+    if (pos_table && (!positions || npos <= 0)) return tli_fail("embed: a position table needs positions");
+    hipStream_t s = (hipStream_t)stream;
+    if (dtype == TLI_F32)
+        embed_scaled_kernel<float><<<rows, 256, 0, s>>>((const float*)table, ids, (const float*)pos_table, positions,
+                                                        out, hidden, vocab, npos, scale);
+    else if (dtype == TLI_BF16)
+        embed_scaled_kernel<bf16_t><<<rows, 256, 0, s>>>((const bf16_t*)table, ids, (const bf16_t*)pos_table,
+                                                         positions, out, hidden, vocab, npos, scale);
+    else
+        return tli_fail("embed: unknown dtype %d", dtype);
+    return tli_check_launch("embed_scaled");
+}
+
+// Activations of a feed-forward without a gate, element by element in float32:
+// 0 relu(z)^2, 1 relu(z), 2 z / (1 + exp(-z)), 3 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3)))
+#define TLI_ACT_KINDS 4
+__device__ __forceinline__ float act_of(float z, int kind) {
+    switch (kind) {
+        case 0: { const float r = fmaxf(z, 0.f); return r * r; }
+        case 1: return fmaxf(z, 0.f);
+        case 2: return z / (1.0f + expf(-z));
+        default: return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+    }
+}
+
+template <typename T>
+__global__ void activation_kernel(const T* __restrict__ x, T* __restrict__ out, size_t total, int kind) {
+    const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx < total) from_f32(out + idx, act_of(to_f32(x[idx]), kind));
+}
+
+// 8 elements a thread, 16-byte loads and stores (total % 8 == 0, both pointers 16-byte aligned)
+__global__ void activation_vec_kernel(const bf16_t* __restrict__ x, bf16_t* __restrict__ out, size_t groups, int kind) {
+    const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= groups) return;
+    const uint4 v = *reinterpret_cast<const uint4*>(x + idx * 8);
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+    uint32_t o[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        o[i] = pack_bf16x2(act_of(__uint_as_float(w[i] << 16), kind), act_of(__uint_as_float(w[i] & 0xFFFF0000u), kind));
+    *reinterpret_cast<uint4*>(out + idx * 8) = make_uint4(o[0], o[1], o[2], o[3]);
+}
+
+extern "C" int tli_activation(const void* x, void* out, long long total, int kind, int dtype, void* stream) {
+    if (total <= 0) return 0;
+    if (kind < 0 || kind >= TLI_ACT_KINDS) return tli_fail("activation: unknown kind %d", kind);
+    hipStream_t s = (hipStream_t)stream;
+    const size_t n = (size_t)total;
+    if (dtype == TLI_F32)
+        activation_kernel<float><<<(unsigned)((n + 255) / 256), 256, 0, s>>>((const float*)x, (float*)out, n, kind);
+    else if (dtype == TLI_BF16 && n % 8 == 0 && !(((uintptr_t)x | (uintptr_t)out) & 15))
+        activation_vec_kernel<<<(unsigned)((n / 8 + 255) / 256), 256, 0, s>>>((const bf16_t*)x, (bf16_t*)out, n / 8, kind);
+    else if (dtype == TLI_BF16)
+        activation_kernel<bf16_t><<<(unsigned)((n + 255) / 256), 256, 0, s>>>((const bf16_t*)x, (bf16_t*)out, n, kind);
+    else
+        return tli_fail("activation: unknown dtype %d", dtype);
+    return tli_check_launch("activation");
+}
+
+// z <- cap * tanh(z / cap), float32, in place
+__global__ void softcap_kernel(float* __restrict__ z, size_t total, float cap) {
+    const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx < total) z[idx] = cap * tanhf(z[idx] / cap);
+}
+
+extern "C" int tli_softcap(float* z, long long total, float cap, void* stream) {
+    if (total <= 0) return 0;
+    if (!(cap > 0.f)) return tli_fail("softcap: the cap must be positive");
+    softcap_kernel<<<(unsigned)(((size_t)total + 255) / 256), 256, 0, (hipStream_t)stream>>>(z, (size_t)total, cap);
+    return tli_check_launch("softcap");
+}

@@ -1,0 +1,203 @@
+// Several copies of the residual stream side by side (hyper-connections), and the token shift.
+//
+// The residual is float32 [rows][S][n].  A sublayer that read u = sum_s in[s] x_s and gave y is
+// written back as x_t <- sum_s mix[s][t] x_s + out[t] y, every stream from the old ones.
+//
+// streams_open:  x[r][s][:] = e[r][:] for every s.
+// streams_norm:  one workgroup a row: (1) if a sublayer's y is still owed, the streams are
+//                rewritten as above; (2) u = sum_s in[s] x_s of the new streams; (3)
+//                h = w * u / sqrt(mean(u^2) + eps).  With a list of rows only those are computed
+//                and the streams are left as they are (the last norm of a step, with in = 1: the
+//                streams' sum).  All arithmetic is float32; u is kept in LDS between the passes.
+//                With a shift (steps of one row a sequence): h is mixed with the sequence's
+//                kept row and replaces it, as token_shift does.
+// token_shift:   out[r] = h[r] + (prev - h[r]) * mu, prev the row before of the same sequence:
+//                in this step, or the kept row of the sequence's slot (nothing at position 0).
+//                The workgroup of a sequence's first row, having read the kept row, replaces it
+//                by the sequence's last row of this step: each element is read and written by
+//                the same thread.
+#include "common.h"
+
+#define ST_MAX_STREAMS 8
+#define ST_MAX_WIDTH 15360          // a row of u in LDS: 60 KiB
+
+__global__ void streams_open_kernel(const float* __restrict__ e, float* __restrict__ x, int n, int S) {
+    const size_t row = blockIdx.x;
+    for (int i = threadIdx.x; i < n; i += blockDim.x) {
+        const float v = e[row * n + i];
+        for (int s = 0; s < S; ++s) x[(row * S + s) * n + i] = v;
+    }
+}
+
+extern "C" int tli_streams_open(const float* e, float* x, int rows, int n, int streams, void* stream) {
+    if (rows <= 0) return 0;
+    if (n <= 0 || streams <= 0) return tli_fail("streams_open: bad sizes n=%d streams=%d", n, streams);
+    streams_open_kernel<<<rows, 256, 0, (hipStream_t)stream>>>(e, x, n, streams);
+    return tli_check_launch("streams_open");
+}
+
+struct ShiftArgs {
+    const float* mu;          // null: no shift
+    float* kept;              // [slots][n]
+    const int* slots;         // [seqs]
+    const int* seq_start;     // [seqs]
+    const int* seq_of_row;    // [rows]
+};
+
+template <typename TD, typename TO, int S>
+__global__ void streams_norm_kernel(float* __restrict__ resid, const TD* __restrict__ delta,
+                                    const float* __restrict__ mix, const float* __restrict__ out_w,
+                                    const float* __restrict__ in_w, const float* __restrict__ weight,
+                                    TO* __restrict__ out, const int* __restrict__ rows, int n, float eps,
+                                    int total_rows, ShiftArgs sh) {
+    extern __shared__ float u_s[];
+    __shared__ float scratch[16];
+    const int out_row = blockIdx.x;
+    int r = rows ? rows[out_row] : out_row;
+    if (r < 0 || r >= total_rows) r = 0;
+    float* x = resid + (size_t)r * S * n;
+    const bool owed = delta != nullptr;
+    const bool update = owed && rows == nullptr;
+    float m[S][S], o[S], a[S];
+#pragma unroll
+    for (int s = 0; s < S; ++s) {
+        a[s] = in_w[s];
+        o[s] = owed ? out_w[s] : 0.f;
+#pragma unroll
+        for (int t = 0; t < S; ++t) m[s][t] = owed ? mix[s * S + t] : 0.f;
+    }
+    const TD* y_row = owed ? delta + (size_t)r * n : nullptr;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < n; i += blockDim.x) {
+        float xs[S];
+#pragma unroll
+        for (int s = 0; s < S; ++s) xs[s] = x[(size_t)s * n + i];
+        if (owed) {
+            const float y = to_f32(y_row[i]);
+            float xn[S];
+#pragma unroll
+            for (int t = 0; t < S; ++t) {
+                float acc = 0.f;
+#pragma unroll
+                for (int s = 0; s < S; ++s) acc += m[s][t] * xs[s];
+                xn[t] = acc + o[t] * y;
+            }
+#pragma unroll
+            for (int t = 0; t < S; ++t) {
+                xs[t] = xn[t];
+                if (update) x[(size_t)t * n + i] = xn[t];
+            }
+        }
+        float u = 0.f;
+#pragma unroll
+        for (int s = 0; s < S; ++s) u += a[s] * xs[s];
+        u_s[i] = u;
+        ss += u * u;
+    }
+    ss = block_sum(ss, scratch);
+    const float scale = 1.0f / sqrtf(ss / (float)n + eps);
+    TO* dst = out + (size_t)out_row * n;
+    if (sh.mu == nullptr) {
+        for (int i = threadIdx.x; i < n; i += blockDim.x) from_f32(dst + i, weight[i] * u_s[i] * scale);
+        return;
+    }
+    const int seq = sh.seq_of_row[r];
+    float* kept = sh.kept + (size_t)sh.slots[seq] * n;
+    const bool fresh = sh.seq_start[seq] <= 0;
+    for (int i = threadIdx.x; i < n; i += blockDim.x) {
+        const float h = weight[i] * u_s[i] * scale;
+        const float prev = fresh ? 0.f : kept[i];
+        kept[i] = h;
+        from_f32(dst + i, h + (prev - h) * sh.mu[i]);
+    }
+}
+
+template <typename TD, typename TO, int S>
+static void launch_streams_norm_s(float* resid, const void* delta, const float* mix, const float* out_w, const float* in_w,
+                                  const float* weight, void* out, const int* rows, int out_rows, int total_rows, int n,
+                                  float eps, ShiftArgs sh, hipStream_t s) {
+    const int threads = n >= 2048 ? 512 : 256;
+    streams_norm_kernel<TD, TO, S><<<out_rows, threads, (size_t)n * sizeof(float), s>>>(
+        resid, (const TD*)delta, mix, out_w, in_w, weight, (TO*)out, rows, n, eps, total_rows, sh);
+}
+
+template <typename TD, typename TO>
+static int launch_streams_norm(int S, float* resid, const void* delta, const float* mix, const float* out_w,
+                               const float* in_w, const float* weight, void* out, const int* rows, int out_rows,
+                               int total_rows, int n, float eps, ShiftArgs sh, hipStream_t s) {
+#define ST_CASE(N) case N: launch_streams_norm_s<TD, TO, N>(resid, delta, mix, out_w, in_w, weight, out, rows, out_rows, total_rows, n, eps, sh, s); break;
+    switch (S) {
+        ST_CASE(1) ST_CASE(2) ST_CASE(3) ST_CASE(4) ST_CASE(5) ST_CASE(6) ST_CASE(7) ST_CASE(8)
+        default: return tli_fail("streams_norm: %d streams, at most %d", S, ST_MAX_STREAMS);
+    }
+#undef ST_CASE
+    return 0;
+}
+
+// delta_dtype: of the owed rows y [total_rows][n] (ignored without them); out_dtype: of the normed rows.
+// mu != null: the shift for steps of one row a sequence (rows must be null).
+extern "C" int tli_streams_norm(float* resid, const void* delta, const float* mix, const float* out_w,
+                                const float* in_w, const float* weight, void* out, const int* rows, int out_rows,
+                                int total_rows, int n, int streams, float eps, int delta_dtype, int out_dtype,
+                                const float* mu, float* kept, const int* slots, const int* seq_start,
+                                const int* seq_of_row, void* stream) {
+    if (out_rows <= 0) return 0;
+    if (n <= 0 || n > ST_MAX_WIDTH) return tli_fail("streams_norm: row size %d is outside 1..%d", n, ST_MAX_WIDTH);
+    if (delta && (!mix || !out_w)) return tli_fail("streams_norm: owed rows need their mix and out weights");
+    if (mu && (rows || !kept || !slots || !seq_start || !seq_of_row))
+        return tli_fail("streams_norm: the shift takes every row of a step and the sequences' slots");
+    if (!delta) delta_dtype = out_dtype == TLI_F32 ? TLI_F32 : TLI_BF16;
+    const ShiftArgs sh{mu, kept, slots, seq_start, seq_of_row};
+    hipStream_t s = (hipStream_t)stream;
+    int rc;
+    if (delta_dtype == TLI_F32 && out_dtype == TLI_F32)
+        rc = launch_streams_norm<float, float>(streams, resid, delta, mix, out_w, in_w, weight, out, rows, out_rows, total_rows, n, eps, sh, s);
+    else if (delta_dtype == TLI_BF16 && out_dtype == TLI_BF16)
+        rc = launch_streams_norm<bf16_t, bf16_t>(streams, resid, delta, mix, out_w, in_w, weight, out, rows, out_rows, total_rows, n, eps, sh, s);
+    else if (delta_dtype == TLI_BF16 && out_dtype == TLI_F32)
+        rc = launch_streams_norm<bf16_t, float>(streams, resid, delta, mix, out_w, in_w, weight, out, rows, out_rows, total_rows, n, eps, sh, s);
+    else
+        return tli_fail("streams_norm: owed rows of dtype %d with normed rows of dtype %d", delta_dtype, out_dtype);
+    if (rc) return rc;
+    return tli_check_launch("streams_norm");
+}
+
+template <typename TO>
+__global__ void token_shift_kernel(const float* __restrict__ h, const float* __restrict__ mu, float* __restrict__ kept,
+                                   TO* __restrict__ out, const int* __restrict__ seq_of_row,
+                                   const int* __restrict__ row_start, const int* __restrict__ seq_start,
+                                   const int* __restrict__ slots, int n) {
+    const int r = blockIdx.x;
+    const int seq = seq_of_row[r];
+    const int first = row_start[seq], last = row_start[seq + 1] - 1;
+    const float* cur = h + (size_t)r * n;
+    TO* dst = out + (size_t)r * n;
+    if (r > first) {
+        const float* before = h + (size_t)(r - 1) * n;
+        for (int i = threadIdx.x; i < n; i += blockDim.x) from_f32(dst + i, cur[i] + (before[i] - cur[i]) * mu[i]);
+        return;
+    }
+    float* k = kept + (size_t)slots[seq] * n;
+    const float* end = h + (size_t)last * n;
+    const bool fresh = seq_start[seq] <= 0;
+    for (int i = threadIdx.x; i < n; i += blockDim.x) {
+        const float prev = fresh ? 0.f : k[i];
+        k[i] = end[i];
+        from_f32(dst + i, cur[i] + (prev - cur[i]) * mu[i]);
+    }
+}
+
+extern "C" int tli_token_shift(const float* h, const float* mu, float* kept, void* out, const int* seq_of_row,
+                               const int* row_start, const int* seq_start, const int* slots, int rows, int n,
+                               int out_dtype, void* stream) {
+    if (rows <= 0) return 0;
+    if (n <= 0) return tli_fail("token_shift: bad row size %d", n);
+    hipStream_t s = (hipStream_t)stream;
+    if (out_dtype == TLI_F32)
+        token_shift_kernel<float><<<rows, 256, 0, s>>>(h, mu, kept, (float*)out, seq_of_row, row_start, seq_start, slots, n);
+    else if (out_dtype == TLI_BF16)
+        token_shift_kernel<bf16_t><<<rows, 256, 0, s>>>(h, mu, kept, (bf16_t*)out, seq_of_row, row_start, seq_start, slots, n);
+    else
+        return tli_fail("token_shift: unknown dtype %d", out_dtype);
+    return tli_check_launch("token_shift");
+}

@@ -315,15 +315,18 @@ class ModelRunner:
         key = (view.num_seqs, view.groups[0].table_width if view.groups else 0, view.reach, view.skew)
         entry = self.graphs.get(key)
         if entry is None:
-            self.forward(view, wanted)                 # once eagerly: anything lazy happens now
+            # The first step of a shape runs eagerly (anything lazy happens now) and its result is the
+            # step's result; the launch sequence is then recorded for the steps to come, which runs
+            # nothing.  (A block that keeps state per request must see every step exactly once.)
+            result = self.forward(view, wanted)
             torch.cuda.synchronize(self.env.device)
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph, pool=self.graph_pool):
                 out = self.forward(view, wanted)
             if self.graph_pool is None:
                 self.graph_pool = graph.pool()
-            entry = (graph, out)
-            self.graphs[key] = entry
+            self.graphs[key] = (graph, out)
+            return result
         entry[0].replay()
         self.graph_replays += 1
         return entry[1]

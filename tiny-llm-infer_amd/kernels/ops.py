@@ -94,6 +94,14 @@ def load_library():
                                           F, I, I, I, P, I, P],
         "tli_attention_prefill_bf16": [P, P, P, P, P, P, I, I, P, I, I, I, I, I, I, F, I, I, P],
         "tli_qkv_attention_prefill_bf16": [P, P, P, P, P, P, I, I, P, I, I, I, I, I, I, P, F, P, P, F, I, I, P],
+        "tli_embed_scaled": [P, P, P, P, P, I, I, I, I, F, I, P],
+        "tli_activation": [P, P, ctypes.c_longlong, I, I, P],
+        "tli_softcap": [P, ctypes.c_longlong, F, P],
+        "tli_streams_open": [P, P, I, I, I, P],
+        "tli_streams_norm": [P, P, P, P, P, P, P, P, I, I, I, I, F, I, I, P, P, P, P, P, P],
+        "tli_token_shift": [P, P, P, P, P, P, P, P, I, I, I, P],
+        "tli_conv_heads": [P, P, P, P, P, P, P, P, P, P, I, I, P, I, I, I, I, I, I, I, I, P],
+        "tli_attention_biased_plain": [P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, P, P, P, I, I, I, P],
         "tli_sample": [P, I, I, P, P, P, P, P, P],
         "tli_sample_scratch_bytes": [I],
         "tli_random_normal": [P, ctypes.c_longlong, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint32, P, F, F, I, P],
@@ -250,13 +258,26 @@ class HipOps:
         self._call(self.lib.tli_feed_tokens, token_ids.data_ptr(), token_from.data_ptr(), src.data_ptr(),
                    rows, src.numel(), self._stream())
 
-    def embed(self, table: torch.Tensor, token_ids: torch.Tensor, num_rows: int) -> torch.Tensor:
+    def embed(self, table: torch.Tensor, token_ids: torch.Tensor, num_rows: int, scale: float = 1.0,
+              positions: Optional[torch.Tensor] = None, pos_table: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """float32 rows [num_rows, hidden]: table[id], or scale * table[id] + pos_table[position]."""
         vocab, hidden = table.shape
         self._want(table, "embedding table")
         self._want(token_ids, "token ids", torch.int32)
         if token_ids.numel() < num_rows:
             raise KernelError("fewer token ids than rows")
         out = torch.empty((num_rows, hidden), dtype=torch.float32, device=self.device)
+        if pos_table is not None or scale != 1.0:
+            npos = 0
+            if pos_table is not None:
+                npos = pos_table.shape[0]
+                self._want(pos_table, "position table", table.dtype, (npos, hidden))
+                self._want(positions, "positions", torch.int32)
+                if positions.numel() < num_rows:
+                    raise KernelError("fewer positions than rows")
+            self._call(self.lib.tli_embed_scaled, table.data_ptr(), token_ids.data_ptr(), _ptr(pos_table), _ptr(positions),
+                       out.data_ptr(), num_rows, hidden, vocab, npos, float(scale), _dtype_code(table.dtype), self._stream())
+            return out
         self._call(self.lib.tli_embed, table.data_ptr(), token_ids.data_ptr(), out.data_ptr(),
                    num_rows, hidden, vocab, _dtype_code(table.dtype), self._stream())
         return out
@@ -824,6 +845,160 @@ class HipOps:
                    kc.data_ptr(), vc.data_ptr(), step.positions.data_ptr(), step.seq_of_row.data_ptr(),
                    g.tables.data_ptr(), g.table_width, g.page_size, kc.shape[0], T, heads, kv_heads,
                    head_dim, float(scale), int(window or 0), splits, per_split, self._stream())
+        return out
+
+    # ---- feed-forward without a gate, soft cap -----------------------------------------
+    ACTIVATIONS = {"relu2": 0, "relu": 1, "silu": 2, "gelu_tanh": 3}
+
+    def check_activation(self, name: str) -> None:
+        if name not in self.ACTIVATIONS:
+            raise KernelError(f"activation '{name}' is not known; known: {', '.join(sorted(self.ACTIVATIONS))}")
+
+    def activation(self, x: torch.Tensor, name: str) -> torch.Tensor:
+        self.check_activation(name)
+        self._want(x, "activation input")
+        out = torch.empty_like(x)
+        self._call(self.lib.tli_activation, x.data_ptr(), out.data_ptr(), x.numel(), self.ACTIVATIONS[name],
+                   _dtype_code(x.dtype), self._stream())
+        return out
+
+    def softcap(self, logits: torch.Tensor, cap: float) -> torch.Tensor:
+        """logits <- cap * tanh(logits / cap), in place (float32)."""
+        self._want(logits, "logits", torch.float32)
+        self._call(self.lib.tli_softcap, logits.data_ptr(), logits.numel(), float(cap), self._stream())
+        return logits
+
+    # ---- several residual streams (hyper-connections), token shift ---------------------------
+    MAX_STREAMS = 8
+    MAX_STREAM_WIDTH = 15360
+
+    def check_streams(self, streams: int, width: int) -> None:
+        if not 1 <= streams <= self.MAX_STREAMS or not 1 <= width <= self.MAX_STREAM_WIDTH:
+            raise KernelError(f"{streams} residual streams of width {width}: the kernels take up to "
+                              f"{self.MAX_STREAMS} streams of up to {self.MAX_STREAM_WIDTH}")
+
+    def streams_open(self, x: torch.Tensor, streams: int) -> torch.Tensor:
+        rows, n = x.shape
+        self._want(x, "embedding rows", torch.float32)
+        out = torch.empty((rows, streams, n), dtype=torch.float32, device=self.device)
+        self._call(self.lib.tli_streams_open, x.data_ptr(), out.data_ptr(), rows, n, streams, self._stream())
+        return out
+
+    def streams_norm(self, resid, pending, w_in, weight, eps, out_dtype, rows=None, num_rows=None, shift=None):
+        """The streams ``resid`` (float32 [T, S, n]) take what ``pending`` (y with its ``mix`` and
+        ``out`` weights, or None) still owes them; returns norm(sum_s w_in[s] x_s) in ``out_dtype``.
+        With ``rows`` only those rows are computed and the streams stay as they are.  ``shift``
+        (mu, kept rows [slots, n], step): the normed rows are mixed with the row before them
+        (``token_shift``) on their way out."""
+        total, S, n = resid.shape
+        self._want(resid, "residual streams", torch.float32)
+        self._want(weight, "norm weight", torch.float32, (n,))
+        self._want(w_in, "stream read weights", torch.float32, (S,))
+        y = mix = out_w = None
+        if pending is not None:
+            y = self.resolve(pending.y)
+            self._want(y, "owed rows", None, (total, n))
+            mix, out_w = pending.mix, pending.out
+            self._want(mix, "stream mix weights", torch.float32, (S, S))
+            self._want(out_w, "stream write weights", torch.float32, (S,))
+        out_rows = total
+        if rows is not None:
+            if shift is not None:
+                raise KernelError("a token shift takes every row of the step")
+            self._want(rows, "row list", torch.int32)
+            out_rows = rows.numel() if num_rows is None else num_rows
+            if rows.numel() < out_rows:
+                raise KernelError("row list is shorter than the rows asked for")
+        fused = shift is not None and shift[2].max_rows_per_seq == 1 and not self.separate_norms
+        mid_dtype = torch.float32 if (shift is not None and not fused) else out_dtype
+        out = torch.empty((out_rows, n), dtype=mid_dtype, device=self.device)
+        mu = kept = slots = seq_start = seq_of_row = None
+        if fused:
+            mu, kept, step = shift
+            self._check_shift(mu, kept, step, total, n)
+            slots, seq_start, seq_of_row = step.slots, step.seq_start, step.seq_of_row
+        self._call(self.lib.tli_streams_norm, resid.data_ptr(), _ptr(y), _ptr(mix), _ptr(out_w), w_in.data_ptr(),
+                   weight.data_ptr(), out.data_ptr(), _ptr(rows), out_rows, total, n, S, float(eps),
+                   _dtype_code(y.dtype) if y is not None else 0, _dtype_code(mid_dtype), _ptr(mu), _ptr(kept),
+                   _ptr(slots), _ptr(seq_start), _ptr(seq_of_row), self._stream())
+        if shift is not None and not fused:
+            return self.token_shift(out, shift[0], shift[1], shift[2], out_dtype)
+        return out
+
+    def _check_shift(self, mu, kept, step, rows, n):
+        self._want(mu, "shift weights", torch.float32, (n,))
+        self._want(kept, "kept rows of the shift", torch.float32, (kept.shape[0], n))
+        if step.num_rows != rows:
+            raise KernelError(f"the step has {step.num_rows} rows, the shift got {rows}")
+        if max(step.h_slots, default=0) >= kept.shape[0]:
+            raise KernelError("a sequence's slot lies outside the kept rows")
+
+    def token_shift(self, h, mu, kept, step, out_dtype):
+        """out[r] = h[r] + (row before r of its sequence - h[r]) * mu; the row before a step's first
+        row is the sequence's kept row (nothing at position 0), which the sequence's last row replaces."""
+        rows, n = h.shape
+        self._want(h, "rows to shift", torch.float32)
+        self._check_shift(mu, kept, step, rows, n)
+        out = torch.empty((rows, n), dtype=out_dtype, device=self.device)
+        self._call(self.lib.tli_token_shift, h.data_ptr(), mu.data_ptr(), kept.data_ptr(), out.data_ptr(),
+                   step.seq_of_row.data_ptr(), step.row_start.data_ptr(), step.seq_start.data_ptr(),
+                   step.slots.data_ptr(), rows, n, _dtype_code(out_dtype), self._stream())
+        return out
+
+    # ---- attention with convolved queries and keys, values = keys ----------------------------
+    MASK_KINDS = {None: 0, "window": 1, "chunk": 2}
+    MAX_CONV_TAPS = 64
+
+    def check_conv_attention_sizes(self, heads: int, kv_heads: int, head_dim: int, taps: int) -> None:
+        if not 1 <= head_dim <= self.MAX_HEAD_DIM:
+            raise KernelError(f"head_dim {head_dim} is not supported: 1 to {self.MAX_HEAD_DIM}")
+        if heads <= 0 or kv_heads <= 0 or heads % kv_heads:
+            raise KernelError(f"{heads} heads cannot be grouped over {kv_heads} kv heads")
+        if not 1 <= taps <= self.MAX_CONV_TAPS:
+            raise KernelError(f"a convolution of {taps} taps is not supported: 1 to {self.MAX_CONV_TAPS}")
+
+    def conv_key_attention(self, qk, bias, conv, state, step, cache, heads, kv_heads, head_dim, taps, scale,
+                           temp, penalty, mask):
+        """From the raw q and k projections [T, (heads + kv_heads) * head_dim] to the attention's
+        output [T, heads * head_dim]: bias, convolution over time (``state``: the sequences' kept
+        rows [slots, taps - 1, channels]), keys into the cache, attention with the keys as values."""
+        T = step.num_rows
+        q_dim, C = heads * head_dim, (heads + kv_heads) * head_dim
+        self.check_conv_attention_sizes(heads, kv_heads, head_dim, taps)
+        self._want(qk, "q and k projections", None, (T, C))
+        self._want(bias, "projection bias", torch.float32, (C,))
+        self._want(conv, "convolution weights", torch.float32, (C, taps))
+        if cache is None or not cache.writes:
+            raise KernelError("this attention writes its keys into a cache layer of its own")
+        kc, g = cache.record("k"), cache.group
+        self._want(kc, "key cache", qk.dtype, (kc.shape[0], kv_heads, g.page_size, head_dim))
+        self._want(g.tables, "block tables", torch.int32, (step.num_seqs, g.table_width))
+        if (step.max_seq_len + g.page_size - 1) // g.page_size > g.table_width:
+            raise KernelError("a block table is narrower than its sequence needs")
+        if taps > 1:
+            if state is None:
+                raise KernelError("the convolution needs the sequences' kept rows")
+            self._want(state, "kept rows of the convolution", qk.dtype, (state.shape[0], taps - 1, C))
+            if max(step.h_slots, default=0) >= state.shape[0]:
+                raise KernelError("a sequence's slot lies outside the kept rows")
+        kind = self.MASK_KINDS.get(mask[0] if mask is not None else None)
+        if kind is None:
+            raise KernelError(f"mask '{mask[0]}' is not known")
+        size = int(mask[1]) if mask is not None else 0
+        r1, r2 = penalty if penalty is not None else (None, None)
+        for w, what in ((temp, "head temperatures"), (r1, "distance penalty"), (r2, "distance penalty")):
+            if w is not None:
+                self._want(w, what, torch.float32, (heads,))
+        q = torch.empty((T, q_dim), dtype=qk.dtype, device=self.device)
+        self._call(self.lib.tli_conv_heads, qk.data_ptr(), bias.data_ptr(), conv.data_ptr(), _ptr(state), q.data_ptr(),
+                   kc.data_ptr(), step.positions.data_ptr(), step.seq_of_row.data_ptr(), step.row_start.data_ptr(),
+                   step.slots.data_ptr(), T, step.num_seqs, g.tables.data_ptr(), g.table_width, g.page_size,
+                   kc.shape[0], heads, kv_heads, head_dim, taps, _dtype_code(qk.dtype), self._stream())
+        out = torch.empty_like(q)
+        self._call(self.lib.tli_attention_biased_plain, q.data_ptr(), out.data_ptr(), kc.data_ptr(), None,
+                   step.positions.data_ptr(), step.seq_of_row.data_ptr(), g.tables.data_ptr(), g.table_width,
+                   g.page_size, kc.shape[0], T, heads, kv_heads, head_dim, float(scale), _ptr(temp), _ptr(r1), _ptr(r2),
+                   kind, size, _dtype_code(qk.dtype), self._stream())
         return out
 
     def sample(self, logits: torch.Tensor, temperatures: Optional[torch.Tensor] = None,
