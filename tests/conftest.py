@@ -20,3 +20,11 @@ def model_folders(tmp_path_factory):
     from helpers import TINY, make_model_folder
     root = tmp_path_factory.mktemp("models")
     return {name: make_model_folder(str(root / name), name) for name in TINY}
+
+
+@pytest.fixture(scope="session")
+def sinepel_folders(tmp_path_factory):
+    """Model folders of the small Sinepel configurations, made once in a temporary folder."""
+    from sinepel_helpers import SMALL, make_folder
+    root = tmp_path_factory.mktemp("sinepel")
+    return {name: make_folder(str(root / name), name) for name in SMALL}

@@ -317,7 +317,8 @@ def test_recorded_decode_steps_equal_eager_ones(model_folders):
                 fast.release(k)
                 slow.release(k)
                 del live[k]
-    assert compared > 30 and fast.graph_replays == compared and len(fast.graphs) >= 3
+    assert compared > 30 and len(fast.graphs) >= 3
+    assert fast.graph_replays == compared - len(fast.graphs)        # (the first step of a shape runs eagerly and is recorded)
 
 
 @pytest.mark.parametrize("first,most,rows,products", [(80, 90, 96, "own"), (140, 150, 160, "own"),
@@ -370,7 +371,7 @@ def test_recorded_steps_of_many_rows_equal_eager_ones(tmp_path, first, most, row
             fast.release(k)
             slow.release(k)
             live.remove(k)
-    assert fast.graph_replays == 14 and {k[0] for k in fast.graphs} == {rows}
+    assert fast.graph_replays == 14 - len(fast.graphs) and {k[0] for k in fast.graphs} == {rows}
 
 
 def test_decode_steps_are_padded_to_few_sizes(model_folders):

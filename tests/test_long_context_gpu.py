@@ -487,7 +487,7 @@ def test_a_long_request_decodes_beside_short_ones(long_request):
     finally:
         type(model.env.ops)._decode_splits = rule
     assert any(skew > 1 and not window and splits > 1 for skew, window, splits in seen), seen[:8]
-    assert runner.graph_replays >= tail - 2
+    assert runner.graph_replays >= tail - 2 - len(runner.graphs)
     for rid, toks in dict(short, r0=reqs["r0"]).items():
         err, row, scale = max_error(got[rid], want[rid][len(toks) - tail:])
         assert err <= 2.5e-2 * scale, f"{rid}: error {err:.3e} at decoded token {row} (logit scale {scale:.3e})"

@@ -415,7 +415,7 @@ def test_many_rows_decoded_together_at_real_width(tmp_path, batch):
             worst = max(worst, float(np.abs(out[i] - w).max() / np.abs(w).max()))
     print(f"{batch} rows decoded together: worst relative error {worst:.2e}")
     assert worst <= TOL["bfloat16"]
-    assert runner.graph_replays == keep
+    assert runner.graph_replays == keep - len(runner.graphs)      # (the first step of a shape runs eagerly and is recorded)
     for rid in ids:
         runner.release(rid)
     runner.cache.check()
