@@ -102,6 +102,7 @@ def load_library():
         "tli_token_shift": [P, P, P, P, P, P, P, P, I, I, I, P],
         "tli_conv_heads": [P, P, P, P, P, P, P, P, P, P, I, I, P, I, I, I, I, I, I, I, I, P],
         "tli_attention_biased_plain": [P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, P, P, P, I, I, I, P],
+        "tli_attention_biased_mfma_bf16": [P, P, P, P, P, P, I, I, P, I, I, I, I, I, I, F, P, P, P, I, I, P],
         "tli_sample": [P, I, I, P, P, P, P, P, P],
         "tli_sample_scratch_bytes": [I],
         "tli_random_normal": [P, ctypes.c_longlong, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint32, P, F, F, I, P],
@@ -995,6 +996,14 @@ class HipOps:
                    step.slots.data_ptr(), T, step.num_seqs, g.tables.data_ptr(), g.table_width, g.page_size,
                    kc.shape[0], heads, kv_heads, head_dim, taps, _dtype_code(qk.dtype), self._stream())
         out = torch.empty_like(q)
+        if qk.dtype == torch.bfloat16 and head_dim % 16 == 0 and head_dim <= 256 and not self.force_plain:
+            starts = step.h_row_start
+            tiles = sum((starts[i + 1] - starts[i] + 15) // 16 for i in range(step.num_seqs))
+            self._call(self.lib.tli_attention_biased_mfma_bf16, q.data_ptr(), out.data_ptr(), kc.data_ptr(), None,
+                       step.row_start.data_ptr(), step.seq_start.data_ptr(), step.num_seqs, tiles, g.tables.data_ptr(),
+                       g.table_width, g.page_size, kc.shape[0], heads, kv_heads, head_dim, float(scale), _ptr(temp),
+                       _ptr(r1), _ptr(r2), kind, size, self._stream())
+            return out
         self._call(self.lib.tli_attention_biased_plain, q.data_ptr(), out.data_ptr(), kc.data_ptr(), None,
                    step.positions.data_ptr(), step.seq_of_row.data_ptr(), g.tables.data_ptr(), g.table_width,
                    g.page_size, kc.shape[0], T, heads, kv_heads, head_dim, float(scale), _ptr(temp), _ptr(r1), _ptr(r2),
