@@ -57,6 +57,93 @@ def step_flops(cfg, layers, rows, ctx_sum, wanted):
     return 2.0 * rows * layers * per_layer + 4.0 * Q * ctx_sum * layers + 2.0 * wanted * V * H
 
 
+DESIGN_SIZES = {
+    # name: width, heads, kv heads, head size, feed-forward, vocabulary
+    "w1024": (1024, 16, 4, 64, 4096, 32768),
+    "w2048": (2048, 16, 4, 128, 8192, 32768),
+    "w4096": (4096, 32, 8, 128, 12288, 32768),
+}
+
+
+def compare_designs(args):
+    """Prefill and decode of the Sinepel design beside the Qwen3 dense decoder at equal layer sizes
+    (random bfloat16 weights, 4 layers unless --layers says otherwise), through the step function:
+    one prompt of --prefill-tokens in one step, and decode steps of --batch and 64 requests at
+    --prompt-len tokens of context.  One JSON line."""
+    import torch
+
+    from tiny_llm_infer_amd.config import Qwen3Config, SinepelConfig
+    from tiny_llm_infer_amd.engine.loading import random_model
+    from tiny_llm_infer_amd.engine.runner import ModelRunner, StepEntry
+    import random
+    rng = random.Random(args.seed)
+    layers = args.layers or 4
+    context = 4096
+    page = 16
+    wanted = [n for n in (args.designs.split(",") if args.designs != "all" else DESIGN_SIZES) if n]
+    points = {}
+    for name in wanted:
+        if name not in DESIGN_SIZES:
+            print(f"--designs {name}: known sizes are {', '.join(DESIGN_SIZES)}")
+            return 2
+        width, heads, kv_heads, dim, ff, vocab = DESIGN_SIZES[name]
+        chunk = 256 if width <= 1024 else 1024
+        sinepel = SinepelConfig.from_dict({
+            "architecture": "Sinepel", "vocab": vocab, "width": width, "max_positions": context, "streams": 4,
+            "embedding": {"scale": 1.0}, "norm": {"eps": 1e-5}, "logit_softcap": 30.0,
+            "layers": [{"type": "attention",
+                        "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "conv": 4,
+                                  "scale": dim ** -0.5, "mask": {"size": chunk}},
+                        "mlp": {"kind": "dense", "ff": ff}}] * layers})
+        qwen = Qwen3Config.from_dict(dict(QWEN3_8B, hidden_size=width, intermediate_size=ff, num_hidden_layers=layers,
+                                          num_attention_heads=heads, num_key_value_heads=kv_heads, head_dim=dim,
+                                          vocab_size=vocab, max_position_embeddings=context))
+        for design, arch, cfg in (("sinepel", "Sinepel", sinepel), ("qwen3", "Qwen3ForCausalLM", qwen)):
+            model = random_model(arch, cfg, args.seed, args.dtype, "cuda:0", context)
+            batches = sorted({args.batch, 64})
+            pages = (args.prefill_tokens + page - 1) // page + max(batches) * ((args.prompt_len + args.steps + args.warmup + 80) // page + 2)
+            runner = ModelRunner(model, model.env, page_size=page, num_pages=pages, max_requests=max(batches) + 1,
+                                 max_batch_tokens=max(args.prefill_tokens, max(batches) * args.prompt_len))
+
+            def timed(fn, n):
+                torch.cuda.synchronize()
+                t = time.perf_counter()
+                for _ in range(n):
+                    fn()
+                torch.cuda.synchronize()
+                return (time.perf_counter() - t) / n
+
+            def prefill():
+                runner.admit("p")
+                runner.step([StepEntry("p", [rng.randrange(vocab) for _ in range(args.prefill_tokens)], [args.prefill_tokens - 1])])
+                runner.release("p")
+            prefill()
+            dt = timed(prefill, 5)
+            points[f"{name}_{design}_prefill_{args.prefill_tokens}"] = {"ms": round(dt * 1e3, 3),
+                                                                   "tokens_per_s": round(args.prefill_tokens / dt, 1)}
+            for batch in batches:
+                keys = [f"d{i}" for i in range(batch)]
+                for k in keys:
+                    runner.admit(k)
+                runner.step([StepEntry(k, [rng.randrange(vocab) for _ in range(args.prompt_len)], []) for k in keys])
+
+                def decode():
+                    runner.step([StepEntry(k, [rng.randrange(vocab)], [0]) for k in keys])
+                for _ in range(args.warmup):
+                    decode()
+                dt = timed(decode, args.steps)
+                for k in keys:
+                    runner.release(k)
+                points[f"{name}_{design}_decode_b{batch}"] = {"ms": round(dt * 1e3, 4), "tokens_per_s": round(batch / dt, 1)}
+            print(f"[bench] {name} {design}: " + ", ".join(f"{k.split('_', 2)[2]} {v['ms']} ms" for k, v in points.items()
+                                                          if k.startswith(f"{name}_{design}_")), file=sys.stderr, flush=True)
+            del runner, model
+            torch.cuda.empty_cache()
+    print(json.dumps({"metric": "design_comparison_tokens_per_s", "unit": "tokens/s", "n_gpus": 1, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+                      "data": "synthetic", "layers": layers, "steps": args.steps, "warmup": args.warmup, "points": points}))
+    return 0
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -83,10 +170,15 @@ def main():
     ap.add_argument("--shape", default=None,
                     help="a config.json whose layer sizes replace the default ones (configs/ holds the larger shapes of the family)")
     ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--designs", default=None,
+                    help="instead of the default workload: the Sinepel design beside the Qwen3 dense decoder at equal layer "
+                         f"sizes, prefill and decode; a list of {','.join(DESIGN_SIZES)} or 'all'")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py runs on one GPU only; --gpus {args.gpus} is not supported (single-GPU engine)")
         return 2
+    if args.designs:
+        return compare_designs(args)
 
     import gc
     import random

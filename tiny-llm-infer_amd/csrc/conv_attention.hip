@@ -20,9 +20,11 @@
 #define CA_MAX_HEAD_DIM 512
 #define CA_MAX_TAPS 64
 
-template <typename T>
+// KEEP: every sequence has one row in this step, and the thread that mixed a channel also moves the
+// sequence's kept rows of that channel up by one and puts the new row last (conv_keep's work).
+template <typename T, bool KEEP>
 __global__ void conv_heads_kernel(const T* __restrict__ qk, const float* __restrict__ bias,
-                                  const float* __restrict__ conv_w, const T* __restrict__ state,
+                                  const float* __restrict__ conv_w, T* __restrict__ state,
                                   T* __restrict__ q_out, T* __restrict__ k_cache,
                                   const int* __restrict__ positions, const int* __restrict__ seq_of_row,
                                   const int* __restrict__ row_start, const int* __restrict__ slots,
@@ -34,7 +36,7 @@ __global__ void conv_heads_kernel(const T* __restrict__ qk, const float* __restr
     const int pos = positions[r];
     const int seq = seq_of_row[r];
     const int first = row_start[seq];
-    const T* kept = state ? state + (size_t)slots[seq] * (taps - 1) * C : nullptr;
+    T* kept = state ? state + (size_t)slots[seq] * (taps - 1) * C : nullptr;
     const float b = bias ? bias[c] : 0.f;
     float acc = 0.f;
     for (int j = 0; j < taps; ++j) {
@@ -45,6 +47,10 @@ __global__ void conv_heads_kernel(const T* __restrict__ qk, const float* __restr
         if (src >= first) u = to_f32(qk[(size_t)src * C + c]);
         else u = to_f32(kept[(size_t)(taps - 1 + src - first) * C + c]);
         acc += conv_w[(size_t)c * taps + j] * (u + b);
+    }
+    if (KEEP && kept) {
+        for (int i = 0; i + 2 < taps; ++i) kept[(size_t)i * C + c] = kept[(size_t)(i + 1) * C + c];
+        kept[(size_t)(taps - 2) * C + c] = qk[(size_t)r * C + c];
     }
     if (c < q_dim) {
         from_f32(q_out + (size_t)r * q_dim + c, acc);
@@ -77,7 +83,7 @@ extern "C" int tli_conv_heads(const void* qk, const float* bias, const float* co
                               void* k_cache, const int* positions, const int* seq_of_row, const int* row_start,
                               const int* slots, int rows, int seqs, const int* tables, int table_width,
                               int page_size, int num_pages, int heads, int kv_heads, int head_dim, int taps,
-                              int dtype, void* stream) {
+                              int one_row_each, int dtype, void* stream) {
     if (rows <= 0) return 0;
     if (heads <= 0 || kv_heads <= 0 || head_dim <= 0) return tli_fail("conv_heads: bad head sizes");
     if (taps <= 0 || taps > CA_MAX_TAPS) return tli_fail("conv_heads: %d taps are outside 1..%d", taps, CA_MAX_TAPS);
@@ -86,16 +92,21 @@ extern "C" int tli_conv_heads(const void* qk, const float* bias, const float* co
     const int q_dim = heads * head_dim, C = q_dim + kv_heads * head_dim;
     hipStream_t s = (hipStream_t)stream;
     const dim3 grid(rows, (C + CA_THREADS - 1) / CA_THREADS), keep(seqs, (C + CA_THREADS - 1) / CA_THREADS);
+    if (one_row_each && rows != seqs) return tli_fail("conv_heads: %d rows of %d sequences are not one row each", rows, seqs);
+#define CA_ARGS(T) (const T*)qk, bias, conv_w, (T*)state, (T*)q_out, (T*)k_cache, positions, seq_of_row, row_start, slots, \
+        tables, table_width, page_size, num_pages, C, q_dim, kv_heads, head_dim, taps
     if (dtype == TLI_F32) {
-        conv_heads_kernel<float><<<grid, CA_THREADS, 0, s>>>(
-            (const float*)qk, bias, conv_w, (const float*)state, (float*)q_out, (float*)k_cache, positions, seq_of_row,
-            row_start, slots, tables, table_width, page_size, num_pages, C, q_dim, kv_heads, head_dim, taps);
-        if (taps > 1) conv_keep_kernel<float><<<keep, CA_THREADS, 0, s>>>((const float*)qk, (float*)state, row_start, slots, C, taps);
+        if (one_row_each) conv_heads_kernel<float, true><<<grid, CA_THREADS, 0, s>>>(CA_ARGS(float));
+        else {
+            conv_heads_kernel<float, false><<<grid, CA_THREADS, 0, s>>>(CA_ARGS(float));
+            if (taps > 1) conv_keep_kernel<float><<<keep, CA_THREADS, 0, s>>>((const float*)qk, (float*)state, row_start, slots, C, taps);
+        }
     } else if (dtype == TLI_BF16) {
-        conv_heads_kernel<bf16_t><<<grid, CA_THREADS, 0, s>>>(
-            (const bf16_t*)qk, bias, conv_w, (const bf16_t*)state, (bf16_t*)q_out, (bf16_t*)k_cache, positions, seq_of_row,
-            row_start, slots, tables, table_width, page_size, num_pages, C, q_dim, kv_heads, head_dim, taps);
-        if (taps > 1) conv_keep_kernel<bf16_t><<<keep, CA_THREADS, 0, s>>>((const bf16_t*)qk, (bf16_t*)state, row_start, slots, C, taps);
+        if (one_row_each) conv_heads_kernel<bf16_t, true><<<grid, CA_THREADS, 0, s>>>(CA_ARGS(bf16_t));
+        else {
+            conv_heads_kernel<bf16_t, false><<<grid, CA_THREADS, 0, s>>>(CA_ARGS(bf16_t));
+            if (taps > 1) conv_keep_kernel<bf16_t><<<keep, CA_THREADS, 0, s>>>((const bf16_t*)qk, (bf16_t*)state, row_start, slots, C, taps);
+        }
     } else {
         return tli_fail("conv_heads: unknown dtype %d", dtype);
     }

@@ -100,7 +100,7 @@ def load_library():
         "tli_streams_open": [P, P, I, I, I, P],
         "tli_streams_norm": [P, P, P, P, P, P, P, P, I, I, I, I, F, I, I, P, P, P, P, P, P],
         "tli_token_shift": [P, P, P, P, P, P, P, P, I, I, I, P],
-        "tli_conv_heads": [P, P, P, P, P, P, P, P, P, P, I, I, P, I, I, I, I, I, I, I, I, P],
+        "tli_conv_heads": [P, P, P, P, P, P, P, P, P, P, I, I, P, I, I, I, I, I, I, I, I, I, P],
         "tli_attention_biased_plain": [P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, P, P, P, I, I, I, P],
         "tli_attention_biased_mfma_bf16": [P, P, P, P, P, P, I, I, P, I, I, I, I, I, I, F, P, P, P, I, I, P],
         "tli_sample": [P, I, I, P, P, P, P, P, P],
@@ -994,7 +994,8 @@ class HipOps:
         self._call(self.lib.tli_conv_heads, qk.data_ptr(), bias.data_ptr(), conv.data_ptr(), _ptr(state), q.data_ptr(),
                    kc.data_ptr(), step.positions.data_ptr(), step.seq_of_row.data_ptr(), step.row_start.data_ptr(),
                    step.slots.data_ptr(), T, step.num_seqs, g.tables.data_ptr(), g.table_width, g.page_size,
-                   kc.shape[0], heads, kv_heads, head_dim, taps, _dtype_code(qk.dtype), self._stream())
+                   kc.shape[0], heads, kv_heads, head_dim, taps,
+                   1 if (step.max_rows_per_seq == 1 and not self.unfused_decode) else 0, _dtype_code(qk.dtype), self._stream())
         out = torch.empty_like(q)
         if qk.dtype == torch.bfloat16 and head_dim % 16 == 0 and head_dim <= 256 and not self.force_plain:
             starts = step.h_row_start
