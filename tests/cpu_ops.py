@@ -101,7 +101,7 @@ class CpuOps:
             else:
                 u = raw[r0:r1] + bias
             n = r1 - r0
-            mixed[r0:r1] = sum(conv[:, j] * u[j:j + n] for j in range(taps))
+            mixed[r0:r1] = sum(conv[j] * u[j:j + n] for j in range(taps))          # conv: [taps, channels]
         q = mixed[:, :qd].to(qk.dtype).to(torch.float32).reshape(T, heads, head_dim)
         k = mixed[:, qd:].reshape(T, kv_heads, head_dim)
         page = cache.group.page_size

@@ -146,7 +146,7 @@ class _Bench:
                         h_row_start=[int(r) for r in row_start], h_seq_start=starts, h_seq_len=totals,
                         h_slots=[rc.slot for rc in rcs], max_rows_per_seq=max(counts), max_seq_len=max(totals),
                         reach=max(128, 1 << (max(totals) - 1).bit_length()), groups=[group])
-        out = ops.conv_key_attention(qk.to(self.dt).cuda(), bias.cuda(), conv.cuda(), self.state, view,
+        out = ops.conv_key_attention(qk.to(self.dt).cuda(), bias.cuda(), conv.t().contiguous().cuda(), self.state, view,
                                      LayerCache(group, 0, True), *self.args, scale, temp, penalty, mask)
         for key in keys:
             self.cm.advance(key, self.cm.get(key).num_tokens + portions[key])

@@ -2,21 +2,13 @@
 // of positions, values from the key cache: the matrix-core kernel for bfloat16 heads whose size is a
 // multiple of 16.  It serves portions of prompts and single decoded rows alike.
 //
-// One wave takes 16 consecutive rows of one sequence (a "tile", counted from the first row that the
-// sequence has in this step) and one head; the four waves of a workgroup take four heads next to each
-// other, which read the same keys where they share a kv head.  Keys are walked 16 at a time from the
-// first one that the tile's first row sees to the tile's last row, each (row, key) pair masked on its own,
-// so a tile may lie across the edge of a block of positions.
+// A workgroup of four waves takes 16 consecutive rows of one sequence (a "tile", counted from the first
+// row that the sequence has in this step) and one head.  The keys from the first one that the tile's first
+// row sees to the tile's last row are walked 16 at a time, the four waves taking every fourth 16 each with
+// sums of their own, which are merged through LDS at the end.  Each (row, key) pair is masked on its own,
+// so a tile may lie across the edge of a block of positions.  A wave brings its 16 keys into LDS with
+// 16-byte loads (a page lookup a lane and pass) and reads both matrix operands from there.
 //
-// Transposed throughout, so that a row's numbers stay in the lanes of one column (lane % 16):
-//   S^T [16 keys x 16 rows]  = K [16 keys x d] . Q^T            A: a key's 4 dims of a lane group, 8 bytes from the cache
-//                                                               B: a row's 4 dims, 8 bytes of q
-//   s = S^T * scale * temp - r1 * ln(1 + r2 * (row position - key position)), float32
-//   weights with a running maximum a row; maxima and sums go over the four lane groups of a column
-//   O^T [d x 16 rows]       += V^T [16 d x 16 keys] . P^T       A: 4 keys of one dim (2-byte loads: the cache keeps
-//                                                               a key's dims together); B: the weights as they lie
-// Lane l of a 16x16x16 tile holds, of A, row l % 16 and k = 4 * (l / 16) .. + 3, of B, column l % 16 and the
-// same k, of the result, column l % 16 and rows 4 * (l / 16) .. + 3.
 #include "common.h"
 
 typedef __attribute__((ext_vector_type(4))) short bf16x4;
@@ -29,11 +21,19 @@ union Frag4 {
 };
 
 #define ABM_WAVES 4
+#define ABM_PAD 8          // bfloat16 elements between the rows of a key tile in LDS (16 bytes: rows stay 16-byte aligned
+                           // and the four lane groups of a gather fall into different banks)
 
 __device__ __forceinline__ int abm_first_visible(int pos, int mask_kind, int mask_size) {
     if (mask_kind == 1) return max(0, pos - mask_size + 1);
     if (mask_kind == 2) return pos - pos % mask_size;
     return 0;
+}
+
+static inline size_t abm_lds_bytes(int D) {
+    const size_t tiles = (size_t)ABM_WAVES * 16 * (D + ABM_PAD) * 2;
+    const size_t merge = (size_t)(ABM_WAVES - 1) * (16 * D + 32) * 4;
+    return tiles > merge ? tiles : merge;
 }
 
 // ND = head_dim / 16.  values: null (the values are the keys) or the value cache [page][kv head][d][slot].
@@ -44,11 +44,11 @@ __global__ __launch_bounds__(64 * ABM_WAVES) void attention_biased_mfma_kernel(
     int num_seqs, const int* __restrict__ tables, int table_width, int page_size, int num_pages, int heads,
     int kv_heads, float scale, const float* __restrict__ temp, const float* __restrict__ r1,
     const float* __restrict__ r2, int mask_kind, int mask_size) {
-    constexpr int D = ND * 16;
-    const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
+    constexpr int D = ND * 16, LD = D + ABM_PAD, CHUNKS = 16 * (D / 8);      // 16-byte pieces of a key tile
+    extern __shared__ __align__(16) unsigned char abm_lds[];
+    const int lane = threadIdx.x % 64, wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
     const int col = lane % 16, grp = lane / 16;
-    const int head = blockIdx.y * ABM_WAVES + wave;
-    if (head >= heads) return;
+    const int head = blockIdx.y;
     // which sequence and which of its tiles
     int tile = blockIdx.x, seq = 0, first_row = 0, count = 0;
     for (; seq < num_seqs; ++seq) {
@@ -58,7 +58,7 @@ __global__ __launch_bounds__(64 * ABM_WAVES) void attention_biased_mfma_kernel(
         if (tile < nt) break;
         tile -= nt;
     }
-    if (seq >= num_seqs) return;
+    if (seq >= num_seqs) return;                                        // (the whole workgroup)
     const int g = head / (heads / kv_heads);
     const int* table = tables + (size_t)seq * table_width;
     const int live = min(16, count - tile * 16);                        // rows of this tile
@@ -81,21 +81,44 @@ __global__ __launch_bounds__(64 * ABM_WAVES) void attention_biased_mfma_kernel(
 #pragma unroll
     for (int j = 0; j < ND; ++j) acc[j] = (f32x4){0.f, 0.f, 0.f, 0.f};
     float m = -INFINITY, l = 0.f;
+    bf16_t* kt = reinterpret_cast<bf16_t*>(abm_lds) + (size_t)wave * 16 * LD;     // this wave's key tile [16][LD]
 
-    for (int k0 = lo - lo % 16; k0 <= hi; k0 += 16) {
-        // A of the scores: key k0 + col, this lane group's dims
-        const int ka = k0 + col;
-        const bf16_t* kp = nullptr;
-        if (ka >= lo && ka <= hi) {
-            const int page = table[ka / page_size];
-            if (page >= 0 && page < num_pages)
-                kp = k_cache + (size_t)page * page_stride + ((size_t)g * page_size + ka % page_size) * D + grp * 4;
+    // A key tile's 16-byte pieces, one a lane and pass: keys outside lo..hi, or without a page, as zeros.  The
+    // loads of the next tile are asked for before the current one is worked on.
+    constexpr int PASSES = (CHUNKS + 63) / 64;
+    uint4 next[PASSES];
+    auto fetch = [&](int k0) {
+#pragma unroll
+        for (int ps = 0; ps < PASSES; ++ps) {
+            const int c = ps * 64 + lane;
+            next[ps] = make_uint4(0, 0, 0, 0);
+            if (CHUNKS % 64 == 0 || c < CHUNKS) {
+                const int key = k0 + c / (D / 8);
+                if (key >= lo && key <= hi) {
+                    const int page = table[key / page_size];
+                    if (page >= 0 && page < num_pages)
+                        next[ps] = *reinterpret_cast<const uint4*>(k_cache + (size_t)page * page_stride +
+                                                                   ((size_t)g * page_size + key % page_size) * D + (c % (D / 8)) * 8);
+                }
+            }
         }
+    };
+    const int k_first = lo - lo % 16 + 16 * wave;
+    if (k_first <= hi) fetch(k_first);
+    for (int k0 = k_first; k0 <= hi; k0 += 16 * ABM_WAVES) {
+#pragma unroll
+        for (int ps = 0; ps < PASSES; ++ps) {
+            const int c = ps * 64 + lane;
+            if (CHUNKS % 64 == 0 || c < CHUNKS)
+                *reinterpret_cast<uint4*>(kt + (c / (D / 8)) * LD + (c % (D / 8)) * 8) = next[ps];
+        }
+        if (k0 + 16 * ABM_WAVES <= hi) fetch(k0 + 16 * ABM_WAVES);
+        wave_lds_sync();
         f32x4 s = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int j = 0; j < ND; ++j) {
             Frag4 a;
-            a.u = kp ? *reinterpret_cast<const uint2*>(kp + j * 16) : make_uint2(0, 0);
+            a.u = *reinterpret_cast<const uint2*>(kt + col * LD + j * 16 + grp * 4);
             s = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a.v, qf[j].v, s, 0, 0, 0);
         }
         // this lane: keys k0 + 4 grp + i of column col
@@ -105,7 +128,7 @@ __global__ __launch_bounds__(64 * ABM_WAVES) void attention_biased_mfma_kernel(
         for (int i = 0; i < 4; ++i) {
             const int key = k0 + grp * 4 + i;
             float v = s[i] * mul;
-            if (r1) v -= pen1 * log1pf(pen2 * (float)(qpos - key));
+            if (r1) v -= pen1 * __logf(1.0f + pen2 * (float)(qpos - key));
             w[i] = (key >= qlo && key <= qpos) ? v : -INFINITY;
             mx = fmaxf(mx, w[i]);
         }
@@ -124,33 +147,80 @@ __global__ __launch_bounds__(64 * ABM_WAVES) void attention_biased_mfma_kernel(
         l = l * corr + quad_rows_sum(sum);
         m = m_new;
         // A of the output: dim 16 j + col of the keys k0 + 4 grp + i
-        const bf16_t* vp[4];
-        size_t vstep;
+        if (v_cache) {
+            const bf16_t* vp[4];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int key = k0 + grp * 4 + i;
-            vp[i] = nullptr;
-            if (key >= lo && key <= hi) {
-                const int page = table[key / page_size];
-                if (page >= 0 && page < num_pages) {
-                    if (v_cache) vp[i] = v_cache + (size_t)page * page_stride + (size_t)g * page_size * D + (size_t)col * page_size + key % page_size;
-                    else vp[i] = k_cache + (size_t)page * page_stride + ((size_t)g * page_size + key % page_size) * D + col;
+            for (int i = 0; i < 4; ++i) {
+                const int key = k0 + grp * 4 + i;
+                vp[i] = nullptr;
+                if (key >= lo && key <= hi) {
+                    const int page = table[key / page_size];
+                    if (page >= 0 && page < num_pages)
+                        vp[i] = v_cache + (size_t)page * page_stride + (size_t)g * page_size * D + (size_t)col * page_size + key % page_size;
                 }
             }
+#pragma unroll
+            for (int j = 0; j < ND; ++j) {
+                Frag4 a;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) a.e[i] = vp[i] ? vp[i][(size_t)j * 16 * page_size] : (bf16_t)0;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) acc[j][i] *= corr;
+                acc[j] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a.v, p.v, acc[j], 0, 0, 0);
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < ND; ++j) {
+                Frag4 a;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) a.e[i] = kt[(grp * 4 + i) * LD + j * 16 + col];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) acc[j][i] *= corr;
+                acc[j] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a.v, p.v, acc[j], 0, 0, 0);
+            }
         }
-        vstep = v_cache ? (size_t)16 * page_size : 16;
+        wave_lds_sync();                                // the tile is read before the next one is written over it
+    }
+    // the four waves' sums into wave 0: each of the others leaves (m, l) a column and its accumulators
+    __syncthreads();
+    float* merge = reinterpret_cast<float*>(abm_lds);
+    constexpr int PER_WAVE = 16 * D + 32;
+    if (wave > 0) {
+        float* mine = merge + (size_t)(wave - 1) * PER_WAVE;
+        if (grp == 0) {
+            mine[col] = m;
+            mine[16 + col] = l;
+        }
+#pragma unroll
+        for (int j = 0; j < ND; ++j)
+            *reinterpret_cast<f32x4*>(mine + 32 + ((size_t)j * 64 + lane) * 4) = acc[j];
+    }
+    __syncthreads();
+    if (wave > 0) return;
+    float mt = m;
+#pragma unroll
+    for (int w = 0; w < ABM_WAVES - 1; ++w) mt = fmaxf(mt, merge[(size_t)w * PER_WAVE + col]);
+    const float f0 = (m == -INFINITY) ? 0.f : __expf(m - mt);
+    float lt = l * f0;
+#pragma unroll
+    for (int j = 0; j < ND; ++j)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[j][i] *= f0;
+#pragma unroll
+    for (int w = 0; w < ABM_WAVES - 1; ++w) {
+        const float* theirs = merge + (size_t)w * PER_WAVE;
+        const float mw = theirs[col];
+        const float f = (mw == -INFINITY) ? 0.f : __expf(mw - mt);
+        lt += theirs[16 + col] * f;
 #pragma unroll
         for (int j = 0; j < ND; ++j) {
-            Frag4 a;
+            const f32x4 a = *reinterpret_cast<const f32x4*>(theirs + 32 + ((size_t)j * 64 + lane) * 4);
 #pragma unroll
-            for (int i = 0; i < 4; ++i) a.e[i] = vp[i] ? vp[i][j * vstep] : (bf16_t)0;
-#pragma unroll
-            for (int i = 0; i < 4; ++i) acc[j][i] *= corr;
-            acc[j] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a.v, p.v, acc[j], 0, 0, 0);
+            for (int i = 0; i < 4; ++i) acc[j][i] += a[i] * f;
         }
     }
     if (col >= live) return;
-    const float inv = l > 0.f ? 1.0f / l : 0.f;
+    const float inv = lt > 0.f ? 1.0f / lt : 0.f;
     bf16_t* o_row = out + ((size_t)(row0 + col) * heads + head) * D;
 #pragma unroll
     for (int j = 0; j < ND; ++j) {
@@ -176,9 +246,10 @@ extern "C" int tli_attention_biased_mfma_bf16(
     if (mask_kind < 0 || mask_kind > 2 || (mask_kind && mask_size <= 0)) return tli_fail("attention: bad mask %d of %d", mask_kind, mask_size);
     if ((r1 == nullptr) != (r2 == nullptr)) return tli_fail("attention: the distance penalty needs both of its numbers");
     if ((((uintptr_t)q | (uintptr_t)out | (uintptr_t)k_cache) & 7)) return tli_fail("attention: operands must be 8-byte aligned");
-    const dim3 grid(tiles, (heads + ABM_WAVES - 1) / ABM_WAVES);
+    if (heads > 65535) return tli_fail("attention: %d heads exceed the grid limit 65535", heads);
+    const dim3 grid(tiles, heads);
     hipStream_t s = (hipStream_t)stream;
-#define ABM_CASE(N) case N: attention_biased_mfma_kernel<N><<<grid, 64 * ABM_WAVES, 0, s>>>( \
+#define ABM_CASE(N) case N: attention_biased_mfma_kernel<N><<<grid, 64 * ABM_WAVES, abm_lds_bytes(16 * N), s>>>( \
         (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)k_cache, (const bf16_t*)v_cache, row_start, seq_start, num_seqs, \
         tables, table_width, page_size, num_pages, heads, kv_heads, scale, temp, r1, r2, mask_kind, mask_size); break;
     switch (head_dim / 16) {

@@ -3,7 +3,8 @@
 //
 // conv_heads:   the raw projections qk [rows][C] (C = q_dim + kv_dim, q first) get their bias and are
 //               mixed over time, channel by channel:
-//                   y[p][c] = sum_j w[c][j] * (qk[p - taps + 1 + j][c] + b[c]),   nothing before position 0.
+//                   y[p][c] = sum_j w[j][c] * (qk[p - taps + 1 + j][c] + b[c]),   nothing before position 0
+//               (w is kept tap by tap, [taps][C], so that neighbouring channels' weights lie together).
 //               Rows before the step's first row of the sequence come from the sequence's kept rows
 //               (state [slots][taps - 1][C], raw projections, oldest first).  The q channels go to
 //               q_out [rows][q_dim], the k channels into the paged cache [page][kv head][slot][d].
@@ -46,7 +47,7 @@ __global__ void conv_heads_kernel(const T* __restrict__ qk, const float* __restr
         float u;
         if (src >= first) u = to_f32(qk[(size_t)src * C + c]);
         else u = to_f32(kept[(size_t)(taps - 1 + src - first) * C + c]);
-        acc += conv_w[(size_t)c * taps + j] * (u + b);
+        acc += conv_w[(size_t)j * C + c] * (u + b);
     }
     if (KEEP && kept) {
         for (int i = 0; i + 2 < taps; ++i) kept[(size_t)i * C + c] = kept[(size_t)(i + 1) * C + c];
@@ -63,6 +64,69 @@ __global__ void conv_heads_kernel(const T* __restrict__ qk, const float* __restr
     from_f32(&v, acc);
     k_cache[(size_t)page * kv_heads * page_size * head_dim + ((size_t)g * page_size + pos % page_size) * head_dim + d] =
         cache_value(v);
+}
+
+
+// The same for bfloat16 with eight channels a thread (16-byte loads and stores): head_dim % 8 == 0.
+template <bool KEEP>
+__global__ void conv_heads_vec_kernel(const bf16_t* __restrict__ qk, const float* __restrict__ bias,
+                                      const float* __restrict__ conv_w, bf16_t* __restrict__ state,
+                                      bf16_t* __restrict__ q_out, bf16_t* __restrict__ k_cache,
+                                      const int* __restrict__ positions, const int* __restrict__ seq_of_row,
+                                      const int* __restrict__ row_start, const int* __restrict__ slots,
+                                      const int* __restrict__ tables, int table_width, int page_size, int num_pages,
+                                      int C, int q_dim, int kv_heads, int head_dim, int taps) {
+    const int r = blockIdx.x;
+    const int c = (blockIdx.y * blockDim.x + threadIdx.x) * 8;
+    if (c >= C) return;
+    const int pos = positions[r];
+    const int seq = seq_of_row[r];
+    const int first = row_start[seq];
+    bf16_t* kept = state ? state + (size_t)slots[seq] * (taps - 1) * C : nullptr;
+    float b[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f}, acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    if (bias) {
+        const float4 b0 = *reinterpret_cast<const float4*>(bias + c), b1 = *reinterpret_cast<const float4*>(bias + c + 4);
+        b[0] = b0.x; b[1] = b0.y; b[2] = b0.z; b[3] = b0.w; b[4] = b1.x; b[5] = b1.y; b[6] = b1.z; b[7] = b1.w;
+    }
+    uint4 newest = make_uint4(0, 0, 0, 0);
+    for (int j = 0; j < taps; ++j) {
+        const int back = taps - 1 - j;
+        if (pos - back < 0) continue;
+        const int src = r - back;
+        const uint4 v = src >= first ? *reinterpret_cast<const uint4*>(qk + (size_t)src * C + c)
+                                     : *reinterpret_cast<const uint4*>(kept + (size_t)(taps - 1 + src - first) * C + c);
+        if (back == 0) newest = v;
+        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+        const float4 t0 = *reinterpret_cast<const float4*>(conv_w + (size_t)j * C + c);
+        const float4 t1 = *reinterpret_cast<const float4*>(conv_w + (size_t)j * C + c + 4);
+        const float t[8] = {t0.x, t0.y, t0.z, t0.w, t1.x, t1.y, t1.z, t1.w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            acc[2 * e] += t[2 * e] * (__uint_as_float(w[e] << 16) + b[2 * e]);
+            acc[2 * e + 1] += t[2 * e + 1] * (__uint_as_float(w[e] & 0xFFFF0000u) + b[2 * e + 1]);
+        }
+    }
+    if (KEEP && kept) {
+        for (int i = 0; i + 2 < taps; ++i)
+            *reinterpret_cast<uint4*>(kept + (size_t)i * C + c) = *reinterpret_cast<const uint4*>(kept + (size_t)(i + 1) * C + c);
+        *reinterpret_cast<uint4*>(kept + (size_t)(taps - 2) * C + c) = newest;
+    }
+    uint32_t o[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const bf16_t lo = cache_value(f32_to_bf16(acc[2 * e])), hi = cache_value(f32_to_bf16(acc[2 * e + 1]));
+        o[e] = (uint32_t)lo | ((uint32_t)hi << 16);
+    }
+    const uint4 y = make_uint4(o[0], o[1], o[2], o[3]);
+    if (c < q_dim) {
+        *reinterpret_cast<uint4*>(q_out + (size_t)r * q_dim + c) = y;
+        return;
+    }
+    const int kc = c - q_dim, g = kc / head_dim, d = kc % head_dim;
+    const int page = tables[(size_t)seq * table_width + pos / page_size];
+    if (page < 0 || page >= num_pages) return;
+    *reinterpret_cast<uint4*>(k_cache + (size_t)page * kv_heads * page_size * head_dim +
+                              ((size_t)g * page_size + pos % page_size) * head_dim + d) = y;
 }
 
 template <typename T>
@@ -100,6 +164,15 @@ extern "C" int tli_conv_heads(const void* qk, const float* bias, const float* co
         else {
             conv_heads_kernel<float, false><<<grid, CA_THREADS, 0, s>>>(CA_ARGS(float));
             if (taps > 1) conv_keep_kernel<float><<<keep, CA_THREADS, 0, s>>>((const float*)qk, (float*)state, row_start, slots, C, taps);
+        }
+    } else if (dtype == TLI_BF16 && head_dim % 8 == 0 &&
+               !(((uintptr_t)qk | (uintptr_t)state | (uintptr_t)q_out | (uintptr_t)k_cache | (uintptr_t)bias | (uintptr_t)conv_w) & 15)) {
+        const int groups = C / 8, threads = groups >= 256 ? 256 : (groups + 63) / 64 * 64;
+        const dim3 vgrid(rows, (groups + threads - 1) / threads);
+        if (one_row_each) conv_heads_vec_kernel<true><<<vgrid, threads, 0, s>>>(CA_ARGS(bf16_t));
+        else {
+            conv_heads_vec_kernel<false><<<vgrid, threads, 0, s>>>(CA_ARGS(bf16_t));
+            if (taps > 1) conv_keep_kernel<bf16_t><<<keep, CA_THREADS, 0, s>>>((const bf16_t*)qk, (bf16_t*)state, row_start, slots, C, taps);
         }
     } else if (dtype == TLI_BF16) {
         if (one_row_each) conv_heads_kernel<bf16_t, true><<<grid, CA_THREADS, 0, s>>>(CA_ARGS(bf16_t));

@@ -112,10 +112,124 @@ __global__ void streams_norm_kernel(float* __restrict__ resid, const TD* __restr
     }
 }
 
+
+// four consecutive elements at once (16-byte aligned float rows, 8-byte aligned bfloat16 rows)
+__device__ __forceinline__ void st_load4(const float* p, float v[4]) {
+    const float4 t = *reinterpret_cast<const float4*>(p);
+    v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+}
+__device__ __forceinline__ void st_load4(const bf16_t* p, float v[4]) {
+    const uint2 t = *reinterpret_cast<const uint2*>(p);
+    v[0] = __uint_as_float(t.x << 16); v[1] = __uint_as_float(t.x & 0xFFFF0000u);
+    v[2] = __uint_as_float(t.y << 16); v[3] = __uint_as_float(t.y & 0xFFFF0000u);
+}
+__device__ __forceinline__ void st_store4(float* p, const float v[4]) {
+    *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+}
+__device__ __forceinline__ void st_store4(bf16_t* p, const float v[4]) {
+    *reinterpret_cast<uint2*>(p) = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+}
+
+// The same, four elements a thread and turn (n % 4 == 0, every row 16-byte aligned).
+template <typename TD, typename TO, int S>
+__global__ void streams_norm_vec_kernel(float* __restrict__ resid, const TD* __restrict__ delta,
+                                        const float* __restrict__ mix, const float* __restrict__ out_w,
+                                        const float* __restrict__ in_w, const float* __restrict__ weight,
+                                        TO* __restrict__ out, const int* __restrict__ rows, int n, float eps,
+                                        int total_rows, ShiftArgs sh) {
+    extern __shared__ __align__(16) float u_s[];
+    __shared__ float scratch[16];
+    const int out_row = blockIdx.x;
+    int r = rows ? rows[out_row] : out_row;
+    if (r < 0 || r >= total_rows) r = 0;
+    float* x = resid + (size_t)r * S * n;
+    const bool owed = delta != nullptr;
+    const bool update = owed && rows == nullptr;
+    float m[S][S], o[S], a[S];
+#pragma unroll
+    for (int s = 0; s < S; ++s) {
+        a[s] = in_w[s];
+        o[s] = owed ? out_w[s] : 0.f;
+#pragma unroll
+        for (int t = 0; t < S; ++t) m[s][t] = owed ? mix[s * S + t] : 0.f;
+    }
+    const TD* y_row = owed ? delta + (size_t)r * n : nullptr;
+    float ss = 0.f;
+    for (int i = threadIdx.x * 4; i < n; i += blockDim.x * 4) {
+        float xs[S][4];
+#pragma unroll
+        for (int s = 0; s < S; ++s) st_load4(x + (size_t)s * n + i, xs[s]);
+        if (owed) {
+            float y[4], xn[S][4];
+            st_load4(y_row + i, y);
+#pragma unroll
+            for (int t = 0; t < S; ++t)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    float acc = 0.f;
+#pragma unroll
+                    for (int s = 0; s < S; ++s) acc += m[s][t] * xs[s][e];
+                    xn[t][e] = acc + o[t] * y[e];
+                }
+#pragma unroll
+            for (int t = 0; t < S; ++t) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) xs[t][e] = xn[t][e];
+                if (update) st_store4(x + (size_t)t * n + i, xn[t]);
+            }
+        }
+        float u[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            u[e] = 0.f;
+#pragma unroll
+            for (int s = 0; s < S; ++s) u[e] += a[s] * xs[s][e];
+            ss += u[e] * u[e];
+        }
+        st_store4(u_s + i, u);
+    }
+    ss = block_sum(ss, scratch);
+    const float scale = 1.0f / sqrtf(ss / (float)n + eps);
+    TO* dst = out + (size_t)out_row * n;
+    const bool shift = sh.mu != nullptr;
+    float* kept = nullptr;
+    bool fresh = true;
+    if (shift) {
+        const int seq = sh.seq_of_row[r];
+        kept = sh.kept + (size_t)sh.slots[seq] * n;
+        fresh = sh.seq_start[seq] <= 0;
+    }
+    for (int i = threadIdx.x * 4; i < n; i += blockDim.x * 4) {
+        float u[4], w[4], h[4];
+        st_load4(u_s + i, u);
+        st_load4(weight + i, w);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) h[e] = w[e] * u[e] * scale;
+        if (shift) {
+            float prev[4] = {0.f, 0.f, 0.f, 0.f}, mu[4];
+            if (!fresh) st_load4(kept + i, prev);
+            st_load4(sh.mu + i, mu);
+            st_store4(kept + i, h);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) h[e] = h[e] + (prev[e] - h[e]) * mu[e];
+        }
+        st_store4(dst + i, h);
+    }
+}
+
 template <typename TD, typename TO, int S>
 static void launch_streams_norm_s(float* resid, const void* delta, const float* mix, const float* out_w, const float* in_w,
                                   const float* weight, void* out, const int* rows, int out_rows, int total_rows, int n,
                                   float eps, ShiftArgs sh, hipStream_t s) {
+    const bool aligned = !(((uintptr_t)resid | (uintptr_t)delta | (uintptr_t)weight | (uintptr_t)out | (uintptr_t)sh.mu |
+                            (uintptr_t)sh.kept) & 15);
+    if (n % 4 == 0 && aligned) {
+        const int groups = n / 4;
+        const int threads = groups >= 512 ? 512 : (groups + 63) / 64 * 64;
+        streams_norm_vec_kernel<TD, TO, S><<<out_rows, threads, (size_t)n * sizeof(float), s>>>(
+            resid, (const TD*)delta, mix, out_w, in_w, weight, (TO*)out, rows, n, eps, total_rows, sh);
+        return;
+    }
     const int threads = n >= 2048 ? 512 : 256;
     streams_norm_kernel<TD, TO, S><<<out_rows, threads, (size_t)n * sizeof(float), s>>>(
         resid, (const TD*)delta, mix, out_w, in_w, weight, (TO*)out, rows, n, eps, total_rows, sh);
@@ -174,6 +288,18 @@ __global__ void token_shift_kernel(const float* __restrict__ h, const float* __r
     TO* dst = out + (size_t)r * n;
     if (r > first) {
         const float* before = h + (size_t)(r - 1) * n;
+        if (n % 4 == 0 && !(((uintptr_t)h | (uintptr_t)mu | (uintptr_t)out) & 15)) {
+            for (int i = threadIdx.x * 4; i < n; i += blockDim.x * 4) {
+                float c[4], b[4], w[4];
+                st_load4(cur + i, c);
+                st_load4(before + i, b);
+                st_load4(mu + i, w);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) c[e] = c[e] + (b[e] - c[e]) * w[e];
+                st_store4(dst + i, c);
+            }
+            return;
+        }
         for (int i = threadIdx.x; i < n; i += blockDim.x) from_f32(dst + i, cur[i] + (before[i] - cur[i]) * mu[i]);
         return;
     }

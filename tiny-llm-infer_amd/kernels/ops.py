@@ -961,14 +961,15 @@ class HipOps:
     def conv_key_attention(self, qk, bias, conv, state, step, cache, heads, kv_heads, head_dim, taps, scale,
                            temp, penalty, mask):
         """From the raw q and k projections [T, (heads + kv_heads) * head_dim] to the attention's
-        output [T, heads * head_dim]: bias, convolution over time (``state``: the sequences' kept
-        rows [slots, taps - 1, channels]), keys into the cache, attention with the keys as values."""
+        output [T, heads * head_dim]: bias, convolution over time (``conv``: its weights tap by tap,
+        [taps, channels], oldest tap first; ``state``: the sequences' kept rows [slots, taps - 1,
+        channels]), keys into the cache, attention with the keys as values."""
         T = step.num_rows
         q_dim, C = heads * head_dim, (heads + kv_heads) * head_dim
         self.check_conv_attention_sizes(heads, kv_heads, head_dim, taps)
         self._want(qk, "q and k projections", None, (T, C))
         self._want(bias, "projection bias", torch.float32, (C,))
-        self._want(conv, "convolution weights", torch.float32, (C, taps))
+        self._want(conv, "convolution weights", torch.float32, (taps, C))
         if cache is None or not cache.writes:
             raise KernelError("this attention writes its keys into a cache layer of its own")
         kc, g = cache.record("k"), cache.group

@@ -80,7 +80,7 @@ class ConvKeyAttention(Mixer):
             return torch.cat([weights[n[r]].to(torch.float32) for r in roles], dim=0).contiguous()
         self.w_qk = fuse_rows([weights[n["q"]], weights[n["k"]]], env)
         self.bias = f32("q_bias", "k_bias")                     # [q_dim + kv_dim]
-        self.conv = f32("q_conv", "k_conv")                     # [q_dim + kv_dim, taps]
+        self.conv = f32("q_conv", "k_conv").t().contiguous()    # [taps, q_dim + kv_dim]: tap by tap, as the kernels read it
         self.temp = f32("temp") if "temp" in n else None
         self.penalty = (f32("r1"), f32("r2")) if "r1" in n else None
         self.w_o = as_matrix(weights[n["o"]], env)
