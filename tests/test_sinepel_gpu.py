@@ -168,10 +168,20 @@ def _plain_mixer_core(raw, bias, conv, heads, kv_heads, dim, scale, temp, r1, r2
     return out
 
 
-@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16", "bfloat16-tiles-of-32"])
 @pytest.mark.parametrize("heads, kv_heads, dim, taps, size, page", [
     (4, 2, 16, 3, 24, 8), (3, 3, 8, 1, 7, 4), (2, 1, 64, 4, 32, 16), (8, 2, 32, 2, 80, 8), (1, 1, 48, 5, 16, 8), (4, 4, 128, 2, 64, 16)])
 def test_mixer_kernels_in_portions_and_decoding(ops, dtype, heads, kv_heads, dim, taps, size, page):
+    if dtype.endswith("32") and dtype != "float32":
+        dtype = "bfloat16"
+        ops.attention_tile_rows = 32
+    try:
+        _mixer_kernels_in_portions_and_decoding(ops, dtype, heads, kv_heads, dim, taps, size, page)
+    finally:
+        ops.attention_tile_rows = 16
+
+
+def _mixer_kernels_in_portions_and_decoding(ops, dtype, heads, kv_heads, dim, taps, size, page):
     """Convolution (with the kept rows), keys into pages, attention inside blocks of positions: two sequences
     in unequal portions, then token by token, against the plain functions on the whole sequences."""
     g = torch.Generator().manual_seed(dim + taps)

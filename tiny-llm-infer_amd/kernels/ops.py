@@ -102,7 +102,7 @@ def load_library():
         "tli_token_shift": [P, P, P, P, P, P, P, P, I, I, I, P],
         "tli_conv_heads": [P, P, P, P, P, P, P, P, P, P, I, I, P, I, I, I, I, I, I, I, I, I, P],
         "tli_attention_biased_plain": [P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, P, P, P, I, I, I, P],
-        "tli_attention_biased_mfma_bf16": [P, P, P, P, P, P, I, I, P, I, I, I, I, I, I, F, P, P, P, I, I, P],
+        "tli_attention_biased_mfma_bf16": [P, P, P, P, P, P, I, I, I, P, I, I, I, I, I, I, F, P, P, P, I, I, P],
         "tli_sample": [P, I, I, P, P, P, P, P, P],
         "tli_sample_scratch_bytes": [I],
         "tli_random_normal": [P, ctypes.c_longlong, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint32, P, F, F, I, P],
@@ -192,6 +192,7 @@ class HipOps:
         self.many_rows = "own"
         self.measured = {}           # (rows rounded up to 128, N, K, gated) -> True where gemm_rows won
         self._cold = None            # what is written between two timed runs
+        self.attention_tile_rows = 16   # measurements, tests: 32 = tiles of 32 rows in the biased attention kernel (heads up to 128)
         self.rows_cfg = 0            # measurements: force a launch shape and the k ranges of gemm_rows
         self.rows_splits = 0
 
@@ -999,10 +1000,13 @@ class HipOps:
                    1 if (step.max_rows_per_seq == 1 and not self.unfused_decode) else 0, _dtype_code(qk.dtype), self._stream())
         out = torch.empty_like(q)
         if qk.dtype == torch.bfloat16 and head_dim % 16 == 0 and head_dim <= 256 and not self.force_plain:
+            # tiles of 16 rows (tiles of 32, two sets of columns a wave sharing each key tile, were measured at
+            # heads of 128 and 2,048 rows in blocks of 1,024 positions: 114 us against 94, fewer waves in flight)
             starts = step.h_row_start
-            tiles = sum((starts[i + 1] - starts[i] + 15) // 16 for i in range(step.num_seqs))
+            per = 32 if (self.attention_tile_rows == 32 and head_dim <= 128) else 16
+            tiles = sum((starts[i + 1] - starts[i] + per - 1) // per for i in range(step.num_seqs))
             self._call(self.lib.tli_attention_biased_mfma_bf16, q.data_ptr(), out.data_ptr(), kc.data_ptr(), None,
-                       step.row_start.data_ptr(), step.seq_start.data_ptr(), step.num_seqs, tiles, g.tables.data_ptr(),
+                       step.row_start.data_ptr(), step.seq_start.data_ptr(), step.num_seqs, tiles, per, g.tables.data_ptr(),
                        g.table_width, g.page_size, kc.shape[0], heads, kv_heads, head_dim, float(scale), _ptr(temp),
                        _ptr(r1), _ptr(r2), kind, size, self._stream())
             return out
