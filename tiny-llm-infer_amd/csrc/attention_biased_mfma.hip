@@ -46,31 +46,35 @@ __global__ __launch_bounds__(64 * ABM_WAVES) void attention_biased_mfma_kernel(
     const bf16_t* __restrict__ v_cache, const int* __restrict__ row_start, const int* __restrict__ seq_start,
     int num_seqs, const int* __restrict__ tables, int table_width, int page_size, int num_pages, int heads,
     int kv_heads, float scale, const float* __restrict__ temp, const float* __restrict__ r1,
-    const float* __restrict__ r2, int mask_kind, int mask_size) {
+    const float* __restrict__ r2, int mask_kind, int mask_size, int grouped) {
     constexpr int D = ND * 16, LD = D + ABM_PAD, CHUNKS = 16 * (D / 8), ROWS = 16 * CT;      // CHUNKS: 16-byte pieces of a key tile
     extern __shared__ __align__(16) unsigned char abm_lds[];
     const int lane = threadIdx.x % 64, wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
     const int col = lane % 16, grp = lane / 16;
-    const int head = blockIdx.y;
+    // grouped > 0 (steps of single rows): a tile is one row, its columns are the `grouped` query heads that share
+    // kv head blockIdx.y, so that a key tile is fetched once for all of them; else blockIdx.y is the query head
+    const int per_tile = grouped ? 1 : ROWS;
     // which sequence and which of its tiles
     int tile = blockIdx.x, seq = 0, first_row = 0, count = 0;
     for (; seq < num_seqs; ++seq) {
         first_row = row_start[seq];
         count = row_start[seq + 1] - first_row;
-        const int nt = (count + ROWS - 1) / ROWS;
+        const int nt = (count + per_tile - 1) / per_tile;
         if (tile < nt) break;
         tile -= nt;
     }
     if (seq >= num_seqs) return;                                        // (the whole workgroup)
-    const int g = head / (heads / kv_heads);
+    const int head = grouped ? blockIdx.y * grouped + min(col, grouped - 1) : blockIdx.y;     // of this lane's column
+    const int g = grouped ? blockIdx.y : head / (heads / kv_heads);
     const int* table = tables + (size_t)seq * table_width;
-    const int live = min(ROWS, count - tile * ROWS);                    // rows of this tile
-    const int row0 = first_row + tile * ROWS;
-    const int pos0 = seq_start[seq] + tile * ROWS;
+    const int live = min(per_tile, count - tile * per_tile);            // rows of this tile
+    const int row0 = first_row + tile * per_tile;
+    const int pos0 = seq_start[seq] + tile * per_tile;
     const int lo = abm_first_visible(pos0, mask_kind, mask_size), hi = pos0 + live - 1;
     const float mul = scale * (temp ? temp[head] : 1.0f);
     const float pen1 = r1 ? r1[head] : 0.f, pen2 = r1 ? r2[head] : 0.f;
     const size_t page_stride = (size_t)kv_heads * page_size * D;
+    const int live_cols = grouped ? grouped : live;                     // columns that are stored
 
     int qpos[CT], qlo[CT];
     Frag4 qf[CT][ND];
@@ -217,7 +221,7 @@ __global__ __launch_bounds__(64 * ABM_WAVES) void attention_biased_mfma_kernel(
     if (wave > 0) return;
 #pragma unroll
     for (int ct = 0; ct < CT; ++ct) {
-        if (ct * 16 >= live) break;
+        if (ct * 16 >= live_cols) break;
         float mt = m[ct];
 #pragma unroll
         for (int w = 0; w < ABM_WAVES - 1; ++w) mt = fmaxf(mt, merge[(size_t)w * PER_WAVE + ct * PER_SET + col]);
@@ -240,9 +244,9 @@ __global__ __launch_bounds__(64 * ABM_WAVES) void attention_biased_mfma_kernel(
                 for (int i = 0; i < 4; ++i) acc[ct][j][i] += a[i] * f;
             }
         }
-        if (ct * 16 + col >= live) continue;
+        if (ct * 16 + col >= live_cols) continue;
         const float inv = lt > 0.f ? 1.0f / lt : 0.f;
-        bf16_t* o_row = out + ((size_t)(row0 + ct * 16 + col) * heads + head) * D;
+        bf16_t* o_row = out + ((size_t)(row0 + (grouped ? 0 : ct * 16 + col)) * heads + head) * D;
 #pragma unroll
         for (int j = 0; j < ND; ++j) {
             uint2 st;
@@ -254,12 +258,13 @@ __global__ __launch_bounds__(64 * ABM_WAVES) void attention_biased_mfma_kernel(
 }
 
 // rows_a_tile: 16 or 32 (heads up to 128 only); tiles: an upper bound of the sum over the sequences of
-// ceil(rows / rows_a_tile) (workgroups past the last tile leave at once)
+// ceil(rows / rows_a_tile) (workgroups past the last tile leave at once).  grouped = heads / kv_heads (at most 16):
+// a tile is one row with the heads of a kv head as its columns, and tiles counts the rows.
 extern "C" int tli_attention_biased_mfma_bf16(
     const void* q, void* out, const void* k_cache, const void* v_cache, const int* row_start, const int* seq_start,
     int num_seqs, int tiles, int rows_a_tile, const int* tables, int table_width, int page_size, int num_pages, int heads,
     int kv_heads, int head_dim, float scale, const float* temp, const float* r1, const float* r2, int mask_kind,
-    int mask_size, void* stream) {
+    int mask_size, int grouped, void* stream) {
     if (num_seqs <= 0 || tiles <= 0) return 0;
     if (head_dim % 16 || head_dim < 16 || head_dim > 256)
         return tli_fail("attention: the matrix-core kernel takes heads of 16 to 256 in steps of 16, not %d", head_dim);
@@ -272,11 +277,13 @@ extern "C" int tli_attention_biased_mfma_bf16(
     if ((r1 == nullptr) != (r2 == nullptr)) return tli_fail("attention: the distance penalty needs both of its numbers");
     if ((((uintptr_t)q | (uintptr_t)out | (uintptr_t)k_cache) & 15)) return tli_fail("attention: operands must be 16-byte aligned");
     if (heads > 65535) return tli_fail("attention: %d heads exceed the grid limit 65535", heads);
-    const dim3 grid(tiles, heads);
+    if (grouped && (grouped != heads / kv_heads || grouped > 16 || rows_a_tile != 16))
+        return tli_fail("attention: %d heads a kv head cannot be one tile's columns", grouped);
+    const dim3 grid(tiles, grouped ? kv_heads : heads);
     hipStream_t s = (hipStream_t)stream;
     const int ct = rows_a_tile / 16;
 #define ABM_ARGS (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)k_cache, (const bf16_t*)v_cache, row_start, seq_start, num_seqs, \
-        tables, table_width, page_size, num_pages, heads, kv_heads, scale, temp, r1, r2, mask_kind, mask_size
+        tables, table_width, page_size, num_pages, heads, kv_heads, scale, temp, r1, r2, mask_kind, mask_size, grouped
 #define ABM_CASE(N) case N: attention_biased_mfma_kernel<N, 1><<<grid, 64 * ABM_WAVES, abm_lds_bytes(16 * N, 1), s>>>(ABM_ARGS); break;
 #define ABM_CASE2(N) case N: if (ct == 2) attention_biased_mfma_kernel<N, 2><<<grid, 64 * ABM_WAVES, abm_lds_bytes(16 * N, 2), s>>>(ABM_ARGS); \
         else attention_biased_mfma_kernel<N, 1><<<grid, 64 * ABM_WAVES, abm_lds_bytes(16 * N, 1), s>>>(ABM_ARGS); break;

@@ -311,6 +311,18 @@ __global__ void embed_scaled_kernel(const T* __restrict__ table, const int* __re
         pv = pos_table + (size_t)p * hidden;
     }
     float* dst = out + (size_t)row * hidden;
+    if (hidden % 4 == 0 && !(((uintptr_t)table | (uintptr_t)pos_table) & 15) && !((uintptr_t)out & 15)) {
+        // four elements a thread and turn
+        for (int i = threadIdx.x * 4; i < hidden; i += blockDim.x * 4) {
+            float e[4], p[4] = {0.f, 0.f, 0.f, 0.f};
+            load4(src + i, e);
+            if (pv) load4(pv + i, p);
+#pragma unroll
+            for (int k = 0; k < 4; ++k) e[k] = scale * e[k] + p[k];
+            store4(dst + i, e);
+        }
+        return;
+    }
     for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
         const float e = scale * to_f32(src[i]);
         dst[i] = pv ? e + to_f32(pv[i]) : e;

@@ -23,6 +23,13 @@
 
 __global__ void streams_open_kernel(const float* __restrict__ e, float* __restrict__ x, int n, int S) {
     const size_t row = blockIdx.x;
+    if (n % 4 == 0 && !(((uintptr_t)e | (uintptr_t)x) & 15)) {
+        for (int i = threadIdx.x * 4; i < n; i += blockDim.x * 4) {
+            const float4 v = *reinterpret_cast<const float4*>(e + row * n + i);
+            for (int s = 0; s < S; ++s) *reinterpret_cast<float4*>(x + (row * S + s) * n + i) = v;
+        }
+        return;
+    }
     for (int i = threadIdx.x; i < n; i += blockDim.x) {
         const float v = e[row * n + i];
         for (int s = 0; s < S; ++s) x[(row * S + s) * n + i] = v;

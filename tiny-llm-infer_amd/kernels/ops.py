@@ -102,7 +102,7 @@ def load_library():
         "tli_token_shift": [P, P, P, P, P, P, P, P, I, I, I, P],
         "tli_conv_heads": [P, P, P, P, P, P, P, P, P, P, I, I, P, I, I, I, I, I, I, I, I, I, P],
         "tli_attention_biased_plain": [P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, P, P, P, I, I, I, P],
-        "tli_attention_biased_mfma_bf16": [P, P, P, P, P, P, I, I, I, P, I, I, I, I, I, I, F, P, P, P, I, I, P],
+        "tli_attention_biased_mfma_bf16": [P, P, P, P, P, P, I, I, I, P, I, I, I, I, I, I, F, P, P, P, I, I, I, P],
         "tli_sample": [P, I, I, P, P, P, P, P, P],
         "tli_sample_scratch_bytes": [I],
         "tli_random_normal": [P, ctypes.c_longlong, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint32, P, F, F, I, P],
@@ -1004,11 +1004,16 @@ class HipOps:
             # heads of 128 and 2,048 rows in blocks of 1,024 positions: 114 us against 94, fewer waves in flight)
             starts = step.h_row_start
             per = 32 if (self.attention_tile_rows == 32 and head_dim <= 128) else 16
-            tiles = sum((starts[i + 1] - starts[i] + per - 1) // per for i in range(step.num_seqs))
+            # single rows (decode steps): the heads of a kv head are one tile's columns and share its keys
+            grouped = heads // kv_heads if (step.max_rows_per_seq == 1 and 1 < heads // kv_heads <= 16
+                                            and not self.unfused_decode) else 0
+            if grouped:
+                per = 16
+            tiles = step.num_rows if grouped else sum((starts[i + 1] - starts[i] + per - 1) // per for i in range(step.num_seqs))
             self._call(self.lib.tli_attention_biased_mfma_bf16, q.data_ptr(), out.data_ptr(), kc.data_ptr(), None,
                        step.row_start.data_ptr(), step.seq_start.data_ptr(), step.num_seqs, tiles, per, g.tables.data_ptr(),
                        g.table_width, g.page_size, kc.shape[0], heads, kv_heads, head_dim, float(scale), _ptr(temp),
-                       _ptr(r1), _ptr(r2), kind, size, self._stream())
+                       _ptr(r1), _ptr(r2), kind, size, grouped, self._stream())
             return out
         self._call(self.lib.tli_attention_biased_plain, q.data_ptr(), out.data_ptr(), kc.data_ptr(), None,
                    step.positions.data_ptr(), step.seq_of_row.data_ptr(), g.tables.data_ptr(), g.table_width,
