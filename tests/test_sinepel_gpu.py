@@ -99,6 +99,17 @@ def test_streams_read_norm_write(ops, streams, dtype):
     _close(got, want[[4, 0, 8]], 2e-5, "rows of a list")
     assert torch.equal(resid2.cpu(), x)
     _close(ops.streams_open(x[:, 0].contiguous().cuda(), S), x[:, :1].expand(T, S, n), 0.0, "opening the streams")
+    if dtype == "bfloat16":
+        # the owed rows as float32 partial sums of a product whose k range was split: added and rounded by the kernel
+        from tiny_llm_infer_amd.kernels.ops import DeferredSum
+        pieces = torch.randn(3, T, n, generator=g)
+        y3 = (pieces[0] + pieces[1] + pieces[2]).to(torch.bfloat16)
+        new3 = plain_sinepel.hyper_write(xs, y3.double(), mix.double(), out_w.double())
+        resid3 = x.clone().cuda()
+        got = ops.streams_norm(resid3, StreamDelta(DeferredSum(pieces.cuda(), torch.bfloat16), mix.cuda(), out_w.cuda()),
+                               in_w.cuda(), weight.cuda(), 1e-5, torch.float32)
+        _close(got, plain_sinepel.rms_norm(plain_sinepel.hyper_read(new3, in_w.double()), weight.double(), 1e-5), 2e-5, "partial sums")
+        _close(resid3, new3.permute(1, 0, 2), 2e-6, "streams after partial sums")
 
 
 class _Bench:
@@ -335,3 +346,45 @@ def test_greedy_generation_through_the_engine(sinepel_folders, dtype):
                 assert float(z.max() - z[t]) <= 2 * TOL["bfloat16"] * float(z.abs().max())
     eng.runner.cache.check()
     assert eng.runner.cache.free_pages() == eng.runner.cache.pages_per_group()
+
+
+# ------------------------------------------------------------------ the command line ---
+def test_the_programs_take_a_sinepel_folder(sinepel_folders, tmp_path):
+    """bin/trace_run replays a mixed trace, model_main --infer generates greedily, and a model of random
+    weights made from a config.json alone (what bench.py --designs runs) loads and generates."""
+    import json
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    folder, vocab = sinepel_folders["Q"], SMALL["Q"][0]["vocab"]
+    reqs = _requests("Q", [40, 9, 77, 23, 52], seed=12)
+    want = plain_logits(folder, reqs)
+    steps = trace_mixed(reqs, max_tokens=192, seed=4)
+    proc = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", folder, "--dtype", "float32",
+                           "--out", str(tmp_path / "out"), "--max-tokens", "192"],
+                          input="".join(json.dumps(s) + "\n" for s in steps), text=True, stdout=subprocess.PIPE,
+                          stderr=subprocess.PIPE, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert proc.stdout.split("\n")[:-1] == [f"done {s['step']}" for s in steps]
+    outputs = {s["step"]: np.fromfile(tmp_path / "out" / f"{s['step']}.f32", dtype="<f4").reshape(-1, vocab)
+               for s in steps if sum(len(e["want"]) for e in s["entries"])}
+    got = collect(steps, outputs)
+    for rid in reqs:
+        err, row, scale = max_error(got[rid], want[rid])
+        assert err <= TOL["float32"] * scale, (rid, err, row)
+    prompt = random_prompt(vocab, 21, 3)
+    proc = subprocess.run([sys.executable, os.path.join(root, "bin", "model_main"), "--infer", "--model", folder, "--dtype",
+                           "float32", "--prompt-ids", ",".join(map(str, prompt)), "--max-new-tokens", "8", "--ignore-eos",
+                           "--max-seq-len", "64", "--num-kv-blocks", "16"],
+                          text=True, stdout=subprocess.PIPE, stderr=subprocess.PIPE, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert [int(t) for t in proc.stdout.split()] == plain_greedy(folder, prompt, 8)
+    cfg_file = tmp_path / "config.json"
+    cfg_file.write_text(json.dumps(SMALL["R"][0]))
+    proc = subprocess.run([sys.executable, os.path.join(root, "bin", "model_main"), "--infer", "--config", str(cfg_file),
+                           "--random-weights", "--seed", "5", "--prompt-ids", "1,2,3,4,5", "--max-new-tokens", "6",
+                           "--ignore-eos", "--max-seq-len", "64", "--num-kv-blocks", "16"],
+                          text=True, stdout=subprocess.PIPE, stderr=subprocess.PIPE, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert len(proc.stdout.split()) == 6

@@ -56,15 +56,17 @@ __global__ void streams_norm_kernel(float* __restrict__ resid, const TD* __restr
                                     const float* __restrict__ mix, const float* __restrict__ out_w,
                                     const float* __restrict__ in_w, const float* __restrict__ weight,
                                     TO* __restrict__ out, const int* __restrict__ rows, int n, float eps,
-                                    int total_rows, ShiftArgs sh) {
+                                    int total_rows, ShiftArgs sh, const float* __restrict__ sums, int parts) {
     extern __shared__ float u_s[];
     __shared__ float scratch[16];
     const int out_row = blockIdx.x;
     int r = rows ? rows[out_row] : out_row;
     if (r < 0 || r >= total_rows) r = 0;
     float* x = resid + (size_t)r * S * n;
-    const bool owed = delta != nullptr;
+    const bool owed = delta != nullptr || parts > 0;
     const bool update = owed && rows == nullptr;
+    const size_t plane = (size_t)total_rows * n;             // of the partial sums [parts][total_rows][n]
+    const float* sum_row = parts > 0 ? sums + (size_t)r * n : nullptr;
     float m[S][S], o[S], a[S];
 #pragma unroll
     for (int s = 0; s < S; ++s) {
@@ -73,14 +75,21 @@ __global__ void streams_norm_kernel(float* __restrict__ resid, const TD* __restr
 #pragma unroll
         for (int t = 0; t < S; ++t) m[s][t] = owed ? mix[s * S + t] : 0.f;
     }
-    const TD* y_row = owed ? delta + (size_t)r * n : nullptr;
+    const TD* y_row = delta ? delta + (size_t)r * n : nullptr;
     float ss = 0.f;
     for (int i = threadIdx.x; i < n; i += blockDim.x) {
         float xs[S];
 #pragma unroll
         for (int s = 0; s < S; ++s) xs[s] = x[(size_t)s * n + i];
         if (owed) {
-            const float y = to_f32(y_row[i]);
+            float y;
+            if (parts > 0) {
+                float a = 0.f;
+                for (int k = 0; k < parts; ++k) a += sum_row[(size_t)k * plane + i];
+                y = bf16_to_f32(f32_to_bf16(a));              // as the product's own reduction would have stored it
+            } else {
+                y = to_f32(y_row[i]);
+            }
             float xn[S];
 #pragma unroll
             for (int t = 0; t < S; ++t) {
@@ -143,15 +152,17 @@ __global__ void streams_norm_vec_kernel(float* __restrict__ resid, const TD* __r
                                         const float* __restrict__ mix, const float* __restrict__ out_w,
                                         const float* __restrict__ in_w, const float* __restrict__ weight,
                                         TO* __restrict__ out, const int* __restrict__ rows, int n, float eps,
-                                        int total_rows, ShiftArgs sh) {
+                                        int total_rows, ShiftArgs sh, const float* __restrict__ sums, int parts) {
     extern __shared__ __align__(16) float u_s[];
     __shared__ float scratch[16];
     const int out_row = blockIdx.x;
     int r = rows ? rows[out_row] : out_row;
     if (r < 0 || r >= total_rows) r = 0;
     float* x = resid + (size_t)r * S * n;
-    const bool owed = delta != nullptr;
+    const bool owed = delta != nullptr || parts > 0;
     const bool update = owed && rows == nullptr;
+    const size_t plane = (size_t)total_rows * n;             // of the partial sums [parts][total_rows][n]
+    const float* sum_row = parts > 0 ? sums + (size_t)r * n : nullptr;
     float m[S][S], o[S], a[S];
 #pragma unroll
     for (int s = 0; s < S; ++s) {
@@ -160,7 +171,7 @@ __global__ void streams_norm_vec_kernel(float* __restrict__ resid, const TD* __r
 #pragma unroll
         for (int t = 0; t < S; ++t) m[s][t] = owed ? mix[s * S + t] : 0.f;
     }
-    const TD* y_row = owed ? delta + (size_t)r * n : nullptr;
+    const TD* y_row = delta ? delta + (size_t)r * n : nullptr;
     float ss = 0.f;
     for (int i = threadIdx.x * 4; i < n; i += blockDim.x * 4) {
         float xs[S][4];
@@ -168,7 +179,19 @@ __global__ void streams_norm_vec_kernel(float* __restrict__ resid, const TD* __r
         for (int s = 0; s < S; ++s) st_load4(x + (size_t)s * n + i, xs[s]);
         if (owed) {
             float y[4], xn[S][4];
-            st_load4(y_row + i, y);
+            if (parts > 0) {
+                float a[4] = {0.f, 0.f, 0.f, 0.f};
+                for (int k = 0; k < parts; ++k) {
+                    float pv[4];
+                    st_load4(sum_row + (size_t)k * plane + i, pv);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) a[e] += pv[e];
+                }
+#pragma unroll
+                for (int e = 0; e < 4; ++e) y[e] = bf16_to_f32(f32_to_bf16(a[e]));      // as the product's own reduction would have stored it
+            } else {
+                st_load4(y_row + i, y);
+            }
 #pragma unroll
             for (int t = 0; t < S; ++t)
 #pragma unroll
@@ -227,26 +250,26 @@ __global__ void streams_norm_vec_kernel(float* __restrict__ resid, const TD* __r
 template <typename TD, typename TO, int S>
 static void launch_streams_norm_s(float* resid, const void* delta, const float* mix, const float* out_w, const float* in_w,
                                   const float* weight, void* out, const int* rows, int out_rows, int total_rows, int n,
-                                  float eps, ShiftArgs sh, hipStream_t s) {
+                                  float eps, ShiftArgs sh, const float* sums, int parts, hipStream_t s) {
     const bool aligned = !(((uintptr_t)resid | (uintptr_t)delta | (uintptr_t)weight | (uintptr_t)out | (uintptr_t)sh.mu |
-                            (uintptr_t)sh.kept) & 15);
+                            (uintptr_t)sh.kept | (uintptr_t)sums) & 15);
     if (n % 4 == 0 && aligned) {
         const int groups = n / 4;
         const int threads = groups >= 512 ? 512 : (groups + 63) / 64 * 64;
         streams_norm_vec_kernel<TD, TO, S><<<out_rows, threads, (size_t)n * sizeof(float), s>>>(
-            resid, (const TD*)delta, mix, out_w, in_w, weight, (TO*)out, rows, n, eps, total_rows, sh);
+            resid, (const TD*)delta, mix, out_w, in_w, weight, (TO*)out, rows, n, eps, total_rows, sh, sums, parts);
         return;
     }
     const int threads = n >= 2048 ? 512 : 256;
     streams_norm_kernel<TD, TO, S><<<out_rows, threads, (size_t)n * sizeof(float), s>>>(
-        resid, (const TD*)delta, mix, out_w, in_w, weight, (TO*)out, rows, n, eps, total_rows, sh);
+        resid, (const TD*)delta, mix, out_w, in_w, weight, (TO*)out, rows, n, eps, total_rows, sh, sums, parts);
 }
 
 template <typename TD, typename TO>
 static int launch_streams_norm(int S, float* resid, const void* delta, const float* mix, const float* out_w,
                                const float* in_w, const float* weight, void* out, const int* rows, int out_rows,
-                               int total_rows, int n, float eps, ShiftArgs sh, hipStream_t s) {
-#define ST_CASE(N) case N: launch_streams_norm_s<TD, TO, N>(resid, delta, mix, out_w, in_w, weight, out, rows, out_rows, total_rows, n, eps, sh, s); break;
+                               int total_rows, int n, float eps, ShiftArgs sh, const float* sums, int parts, hipStream_t s) {
+#define ST_CASE(N) case N: launch_streams_norm_s<TD, TO, N>(resid, delta, mix, out_w, in_w, weight, out, rows, out_rows, total_rows, n, eps, sh, sums, parts, s); break;
     switch (S) {
         ST_CASE(1) ST_CASE(2) ST_CASE(3) ST_CASE(4) ST_CASE(5) ST_CASE(6) ST_CASE(7) ST_CASE(8)
         default: return tli_fail("streams_norm: %d streams, at most %d", S, ST_MAX_STREAMS);
@@ -256,27 +279,33 @@ static int launch_streams_norm(int S, float* resid, const void* delta, const flo
 }
 
 // delta_dtype: of the owed rows y [total_rows][n] (ignored without them); out_dtype: of the normed rows.
+// parts > 0: the owed rows come as float32 partial sums `delta` [parts][total_rows][n] of a product whose k range
+// was split (bfloat16 runs): they are added in order and rounded to bfloat16.
 // mu != null: the shift for steps of one row a sequence (rows must be null).
 extern "C" int tli_streams_norm(float* resid, const void* delta, const float* mix, const float* out_w,
                                 const float* in_w, const float* weight, void* out, const int* rows, int out_rows,
                                 int total_rows, int n, int streams, float eps, int delta_dtype, int out_dtype,
                                 const float* mu, float* kept, const int* slots, const int* seq_start,
-                                const int* seq_of_row, void* stream) {
+                                const int* seq_of_row, int parts, void* stream) {
     if (out_rows <= 0) return 0;
     if (n <= 0 || n > ST_MAX_WIDTH) return tli_fail("streams_norm: row size %d is outside 1..%d", n, ST_MAX_WIDTH);
-    if (delta && (!mix || !out_w)) return tli_fail("streams_norm: owed rows need their mix and out weights");
+    if ((delta || parts > 0) && (!mix || !out_w)) return tli_fail("streams_norm: owed rows need their mix and out weights");
     if (mu && (rows || !kept || !slots || !seq_start || !seq_of_row))
         return tli_fail("streams_norm: the shift takes every row of a step and the sequences' slots");
+    if (parts < 0 || (parts > 0 && (!delta || delta_dtype != TLI_BF16)))
+        return tli_fail("streams_norm: partial sums (%d) go with bfloat16 rows only", parts);
+    const float* sums = parts > 0 ? (const float*)delta : nullptr;
+    if (parts > 0) delta = nullptr;
     if (!delta) delta_dtype = out_dtype == TLI_F32 ? TLI_F32 : TLI_BF16;
     const ShiftArgs sh{mu, kept, slots, seq_start, seq_of_row};
     hipStream_t s = (hipStream_t)stream;
     int rc;
     if (delta_dtype == TLI_F32 && out_dtype == TLI_F32)
-        rc = launch_streams_norm<float, float>(streams, resid, delta, mix, out_w, in_w, weight, out, rows, out_rows, total_rows, n, eps, sh, s);
+        rc = launch_streams_norm<float, float>(streams, resid, delta, mix, out_w, in_w, weight, out, rows, out_rows, total_rows, n, eps, sh, sums, parts, s);
     else if (delta_dtype == TLI_BF16 && out_dtype == TLI_BF16)
-        rc = launch_streams_norm<bf16_t, bf16_t>(streams, resid, delta, mix, out_w, in_w, weight, out, rows, out_rows, total_rows, n, eps, sh, s);
+        rc = launch_streams_norm<bf16_t, bf16_t>(streams, resid, delta, mix, out_w, in_w, weight, out, rows, out_rows, total_rows, n, eps, sh, sums, parts, s);
     else if (delta_dtype == TLI_BF16 && out_dtype == TLI_F32)
-        rc = launch_streams_norm<bf16_t, float>(streams, resid, delta, mix, out_w, in_w, weight, out, rows, out_rows, total_rows, n, eps, sh, s);
+        rc = launch_streams_norm<bf16_t, float>(streams, resid, delta, mix, out_w, in_w, weight, out, rows, out_rows, total_rows, n, eps, sh, sums, parts, s);
     else
         return tli_fail("streams_norm: owed rows of dtype %d with normed rows of dtype %d", delta_dtype, out_dtype);
     if (rc) return rc;

@@ -98,7 +98,7 @@ def load_library():
         "tli_activation": [P, P, ctypes.c_longlong, I, I, P],
         "tli_softcap": [P, ctypes.c_longlong, F, P],
         "tli_streams_open": [P, P, I, I, I, P],
-        "tli_streams_norm": [P, P, P, P, P, P, P, P, I, I, I, I, F, I, I, P, P, P, P, P, P],
+        "tli_streams_norm": [P, P, P, P, P, P, P, P, I, I, I, I, F, I, I, P, P, P, P, P, I, P],
         "tli_token_shift": [P, P, P, P, P, P, P, P, I, I, I, P],
         "tli_conv_heads": [P, P, P, P, P, P, P, P, P, P, I, I, P, I, I, I, I, I, I, I, I, I, P],
         "tli_attention_biased_plain": [P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, P, P, P, I, I, I, P],
@@ -897,9 +897,16 @@ class HipOps:
         self._want(weight, "norm weight", torch.float32, (n,))
         self._want(w_in, "stream read weights", torch.float32, (S,))
         y = mix = out_w = None
+        parts = 0
         if pending is not None:
-            y = self.resolve(pending.y)
-            self._want(y, "owed rows", None, (total, n))
+            y = pending.y
+            if isinstance(y, DeferredSum) and y.dtype == torch.bfloat16 and not self.separate_norms:
+                # partial sums of a split k range: the kernel adds them itself (no pass that only adds)
+                parts, y = y.parts.shape[0], y.parts
+                self._want(y, "partial sums of the owed rows", torch.float32, (parts, total, n))
+            else:
+                y = self.resolve(y)
+                self._want(y, "owed rows", None, (total, n))
             mix, out_w = pending.mix, pending.out
             self._want(mix, "stream mix weights", torch.float32, (S, S))
             self._want(out_w, "stream write weights", torch.float32, (S,))
@@ -921,8 +928,8 @@ class HipOps:
             slots, seq_start, seq_of_row = step.slots, step.seq_start, step.seq_of_row
         self._call(self.lib.tli_streams_norm, resid.data_ptr(), _ptr(y), _ptr(mix), _ptr(out_w), w_in.data_ptr(),
                    weight.data_ptr(), out.data_ptr(), _ptr(rows), out_rows, total, n, S, float(eps),
-                   _dtype_code(y.dtype) if y is not None else 0, _dtype_code(mid_dtype), _ptr(mu), _ptr(kept),
-                   _ptr(slots), _ptr(seq_start), _ptr(seq_of_row), self._stream())
+                   (BF16 if parts else _dtype_code(y.dtype)) if y is not None else 0, _dtype_code(mid_dtype), _ptr(mu), _ptr(kept),
+                   _ptr(slots), _ptr(seq_start), _ptr(seq_of_row), parts, self._stream())
         if shift is not None and not fused:
             return self.token_shift(out, shift[0], shift[1], shift[2], out_dtype)
         return out
