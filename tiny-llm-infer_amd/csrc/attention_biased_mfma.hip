@@ -5,7 +5,7 @@
 // A workgroup of four waves takes 16 consecutive rows of one sequence (a "tile", counted from the first
 // row that the sequence has in this step) and one head.  The keys from the first one that the tile's first
 // row sees to the tile's last row are walked 16 at a time, the four waves taking every fourth 16 each with
-// sums of their own, which are merged through LDS at the end.  Each (row, key) pair is masked on its own,
+// sums of their own, which are merged through LDS at the end (nearest keys first).  Each (row, key) pair is masked on its own,
 // so a tile may lie across the edge of a block of positions.  A wave brings its 16 keys into LDS with
 // 16-byte loads (a page lookup a lane and pass) and reads both matrix operands from there.
 //
@@ -74,6 +74,7 @@ __global__ __launch_bounds__(64 * ABM_WAVES) void attention_biased_mfma_kernel(
     const float mul = scale * (temp ? temp[head] : 1.0f);
     const float pen1 = r1 ? r1[head] : 0.f, pen2 = r1 ? r2[head] : 0.f;
     const size_t page_stride = (size_t)kv_heads * page_size * D;
+    const int page_shift = __builtin_ctz(page_size), page_mask = page_size - 1;      // (a power of two: the launcher checks)
     const int live_cols = grouped ? grouped : live;                     // columns that are stored
 
     int qpos[CT], qlo[CT];
@@ -108,24 +109,26 @@ __global__ __launch_bounds__(64 * ABM_WAVES) void attention_biased_mfma_kernel(
             if (CHUNKS % 64 == 0 || c < CHUNKS) {
                 const int key = k0 + c / (D / 8);
                 if (key >= lo && key <= hi) {
-                    const int page = table[key / page_size];
+                    const int page = table[key >> page_shift];
                     if (page >= 0 && page < num_pages)
                         next[ps] = *reinterpret_cast<const uint4*>(k_cache + (size_t)page * page_stride +
-                                                                   ((size_t)g * page_size + key % page_size) * D + (c % (D / 8)) * 8);
+                                                                   ((size_t)g * page_size + (key & page_mask)) * D + (c % (D / 8)) * 8);
                 }
             }
         }
     };
-    const int k_first = lo - lo % 16 + 16 * wave;
-    if (k_first <= hi) fetch(k_first);
-    for (int k0 = k_first; k0 <= hi; k0 += 16 * ABM_WAVES) {
+    // from the nearest keys to the farthest: with a penalty that grows with the distance the maxima settle in the
+    // first tiles, and the accumulators are rarely rescaled after them
+    const int k_low = lo - lo % 16, k_first = hi - hi % 16 - 16 * wave;
+    if (k_first >= k_low) fetch(k_first);
+    for (int k0 = k_first; k0 >= k_low; k0 -= 16 * ABM_WAVES) {
 #pragma unroll
         for (int ps = 0; ps < PASSES; ++ps) {
             const int c = ps * 64 + lane;
             if (CHUNKS % 64 == 0 || c < CHUNKS)
                 *reinterpret_cast<uint4*>(kt + (c / (D / 8)) * LD + (c % (D / 8)) * 8) = next[ps];
         }
-        if (k0 + 16 * ABM_WAVES <= hi) fetch(k0 + 16 * ABM_WAVES);
+        if (k0 - 16 * ABM_WAVES >= k_low) fetch(k0 - 16 * ABM_WAVES);
         wave_lds_sync();
         // scores: A = the key k0 + col, this lane group's dims, shared by the sets of columns
         f32x4 s[CT];
@@ -168,6 +171,10 @@ __global__ __launch_bounds__(64 * ABM_WAVES) void attention_biased_mfma_kernel(
             l[ct] = l[ct] * corr[ct] + quad_rows_sum(sum);
             m[ct] = m_new;
         }
+        bool moved = false;
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) moved = moved || corr[ct] != 1.0f;
+        const bool rescale = __any(moved);              // (the same for the whole wave)
         // A of the output: dim 16 j + col of the keys k0 + 4 grp + i
         const bf16_t* vp[4] = {nullptr, nullptr, nullptr, nullptr};
         if (v_cache) {
@@ -175,9 +182,9 @@ __global__ __launch_bounds__(64 * ABM_WAVES) void attention_biased_mfma_kernel(
             for (int i = 0; i < 4; ++i) {
                 const int key = k0 + grp * 4 + i;
                 if (key >= lo && key <= hi) {
-                    const int page = table[key / page_size];
+                    const int page = table[key >> page_shift];
                     if (page >= 0 && page < num_pages)
-                        vp[i] = v_cache + (size_t)page * page_stride + (size_t)g * page_size * D + (size_t)col * page_size + key % page_size;
+                        vp[i] = v_cache + (size_t)page * page_stride + (size_t)g * page_size * D + (size_t)col * page_size + (key & page_mask);
                 }
             }
         }
@@ -193,8 +200,10 @@ __global__ __launch_bounds__(64 * ABM_WAVES) void attention_biased_mfma_kernel(
             }
 #pragma unroll
             for (int ct = 0; ct < CT; ++ct) {
+                if (rescale) {
 #pragma unroll
-                for (int i = 0; i < 4; ++i) acc[ct][j][i] *= corr[ct];
+                    for (int i = 0; i < 4; ++i) acc[ct][j][i] *= corr[ct];
+                }
                 acc[ct][j] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a.v, p[ct].v, acc[ct][j], 0, 0, 0);
             }
         }
@@ -273,6 +282,7 @@ extern "C" int tli_attention_biased_mfma_bf16(
     if (heads <= 0 || kv_heads <= 0 || heads % kv_heads)
         return tli_fail("attention: heads %d must be a multiple of kv heads %d", heads, kv_heads);
     if (page_size <= 0 || table_width <= 0 || num_pages <= 0) return tli_fail("attention: bad cache geometry");
+    if (page_size & (page_size - 1)) return tli_fail("attention: the matrix-core kernel takes pages of a power of two, not %d", page_size);
     if (mask_kind < 0 || mask_kind > 2 || (mask_kind && mask_size <= 0)) return tli_fail("attention: bad mask %d of %d", mask_kind, mask_size);
     if ((r1 == nullptr) != (r2 == nullptr)) return tli_fail("attention: the distance penalty needs both of its numbers");
     if ((((uintptr_t)q | (uintptr_t)out | (uintptr_t)k_cache) & 15)) return tli_fail("attention: operands must be 16-byte aligned");
