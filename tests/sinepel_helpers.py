@@ -33,6 +33,10 @@ SMALL = {
     "Q": (_config(131, 48, 1, [_layer(3, 3, 16, 1, 7, 80), _layer(6, 2, 8, 5, 40, 64), _layer(1, 1, 48, 4, 200, 64, scale=0.2)],
                   emb_scale=1.0, eps=3e-6, cap=8.0), 8, 5),
     # four streams, heads of 64 (the matrix-core kernels), one key head for all query heads
+    # three streams, a width that is no multiple of 8, heads of 24 and 20 (no matrix-core attention), eight query
+    # heads on one key head, six taps, blocks of 96, 33 and 50 positions
+    "T": (_config(257, 100, 3, [_layer(6, 3, 24, 6, 96, 144), _layer(2, 2, 20, 2, 33, None), _layer(8, 1, 16, 3, 50, 72)],
+                  emb_scale=0.7, eps=1e-4, cap=30.0), 16, 11),
     "R": (_config(320, 128, 4, [_layer(4, 1, 64, 2, 32, 192), _layer(2, 2, 64, 3, 128, 160)], max_positions=384, cap=12.0), 32, 7),
 }
 
