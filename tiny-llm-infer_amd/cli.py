@@ -282,7 +282,9 @@ def run_replay(argv: List[str], prog: str = "model_main --replay") -> int:
                     help="most tokens live requests hold at any time (each rounded up to 64)")
     ap.add_argument("--page-size", type=int, default=16)
     ap.add_argument("--max-live", type=int, default=4, help="most requests live at a time")
-    ap.add_argument("--max-step-tokens", type=int, default=8192, help="most tokens in one step")
+    ap.add_argument("--max-step-tokens", type=int, default=0,
+                    help="most tokens in one step (0: what --max-live whole requests of the model's longest length "
+                         "bring together, at least 8,192 and at most 262,144)")
     ap.add_argument("--device", default="cuda:0")
     ap.add_argument("--kernels", default="own-products", choices=["own-products", "library-products", "measured", "plain"],
                     help="which kernel multiplies more than 128 rows: this library's (the default: the same "
@@ -301,8 +303,9 @@ def run_replay(argv: List[str], prog: str = "model_main --replay") -> int:
     model = _load(args, None)
     cfg = model.spec.architecture
     pages = max(1, (args.max_tokens + args.page_size - 1) // args.page_size)
+    step_tokens = args.max_step_tokens or min(max(8192, args.max_live * model.spec.max_positions), 1 << 18)
     runner = ModelRunner(model, model.env, page_size=args.page_size, num_pages=pages,
-                         max_requests=args.max_live, max_batch_tokens=args.max_step_tokens)
+                         max_requests=args.max_live, max_batch_tokens=step_tokens)
     print(f"[trace_run] ready: {cfg}, {args.dtype}, {pages} pages of {args.page_size}, "
           f"kernels: {args.kernels}", file=sys.stderr, flush=True)
     Replayer(runner, args.out).run_stream(sys.stdin, ack=sys.stdout)
