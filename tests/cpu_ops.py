@@ -132,6 +132,104 @@ class CpuOps:
                 out[r, h] = torch.softmax(s, dim=0) @ kk[:, h // mul]
         return out.reshape(T, qd).to(qk.dtype)
 
+    # ---- layer norm, the gated delta rule, routed experts ---------------------------------
+    def add_layernorm(self, resid, deltas, weights, eps, out_dtype, rows=None, num_rows=None):
+        owed = None
+        for d in deltas:
+            owed = d.to(torch.float32) if owed is None else owed + d.to(torch.float32)
+        if rows is None:
+            if owed is not None:
+                resid += owed
+            x = resid
+        else:
+            x = resid[rows[:num_rows].long()]
+            if owed is not None:
+                x = x + owed[rows[:num_rows].long()]
+        m = x.mean(dim=-1, keepdim=True)
+        z = (x - m) * torch.rsqrt(((x - m) ** 2).mean(dim=-1, keepdim=True) + eps)
+        return [(z * w).to(out_dtype) for w in weights]
+
+    def check_delta_sizes(self, heads, kv_heads, dk, dv, taps):
+        pass
+
+    def delta_rule(self, proj, gates, conv, a_log, dt_bias, kept, state, step, heads, kv_heads, dk, dv, taps):
+        T = step.num_rows
+        qd, vd = kv_heads * dk, heads * dv
+        C = 2 * qd + vd
+        raw = proj[:, :C].to(torch.float32)
+        out = torch.zeros(T, heads, dv)
+        rep = heads // kv_heads
+        for i in range(step.num_seqs):
+            r0, r1 = step.h_row_start[i], step.h_row_start[i + 1]
+            slot, start, n = step.h_slots[i], step.h_seq_start[i], step.h_row_start[i + 1] - step.h_row_start[i]
+            hist = torch.zeros(taps - 1, C)
+            if taps > 1 and start > 0:
+                hist = kept[slot].to(torch.float32).clone()
+                hist[torch.arange(start - taps + 1, start) < 0] = 0.0
+            u = torch.cat([hist, raw[r0:r1]], dim=0)
+            if taps > 1:
+                kept[slot] = u[-(taps - 1):].to(kept.dtype)
+            c = sum(conv[j] * u[j:j + n] for j in range(taps))
+            c = c / (1 + torch.exp(-c))
+            q = c[:, :qd].reshape(n, kv_heads, dk)
+            k = c[:, qd:2 * qd].reshape(n, kv_heads, dk)
+            v = c[:, 2 * qd:].reshape(n, heads, dv)
+            q = q * torch.rsqrt((q * q).sum(-1, keepdim=True) + 1e-6) * dk ** -0.5
+            k = k * torch.rsqrt((k * k).sum(-1, keepdim=True) + 1e-6)
+            beta = torch.sigmoid(gates[r0:r1, :heads])
+            decay = torch.exp(-torch.exp(a_log) * torch.nn.functional.softplus(gates[r0:r1, heads:] + dt_bias))
+            S = state[slot].clone() if start > 0 else torch.zeros(heads, dk, dv)
+            for t in range(n):
+                kk, qq = k[t].repeat_interleave(rep, 0), q[t].repeat_interleave(rep, 0)      # [H, dk]
+                S = S * decay[t][:, None, None]
+                uu = beta[t][:, None] * (v[t] - torch.einsum("hkv,hk->hv", S, kk))
+                S = S + kk[:, :, None] * uu[:, None, :]
+                out[r0 + t] = torch.einsum("hkv,hk->hv", S, qq)
+            state[slot] = S
+        return out.reshape(T, vd)
+
+    def gated_rmsnorm(self, o, proj, gate_at, weight, eps, heads, dv, out_dtype):
+        T = o.shape[0]
+        x = o.reshape(T, heads, dv)
+        g = proj[:, gate_at:gate_at + heads * dv].to(torch.float32).reshape(T, heads, dv)
+        y = x * torch.rsqrt((x * x).mean(-1, keepdim=True) + eps) * weight * (g / (1 + torch.exp(-g)))
+        return y.reshape(T, heads * dv).to(out_dtype)
+
+    def check_expert_sizes(self, experts, top, groups, keep, hidden, inter):
+        pass
+
+    def pack_experts(self, w_gate_up, w_down):
+        return None
+
+    def route_experts(self, z, experts, top, groups, keep, scale, has_shared):
+        T = z.shape[0]
+        s = torch.sigmoid(z[:, :experts])
+        per = experts // groups
+        score = s.reshape(T, groups, per).topk(min(2, per), dim=-1).values.sum(-1)
+        best = score.topk(keep, dim=-1).indices
+        open_ = torch.zeros(T, groups, dtype=torch.bool)
+        open_.scatter_(1, best, True)
+        masked = torch.where(open_.repeat_interleave(per, 1), s, torch.full_like(s, -1.0))
+        ids = masked.topk(top, dim=-1).indices
+        w = s.gather(1, ids)
+        w = w / (w.sum(-1, keepdim=True) + 1e-20) * scale
+        return ids.to(torch.int32), w, (torch.sigmoid(z[:, experts]) if has_shared else None)
+
+    def apply_experts(self, x, ids, weights, w_gate_up, w_down, packed, shared, shared_gate):
+        T, n = x.shape
+        ff = w_gate_up.shape[1] // 2
+        xf = x.to(torch.float32)
+        out = torch.zeros(T, n)
+        for t in range(T):
+            for j in range(ids.shape[1]):
+                e = int(ids[t, j])
+                gu = w_gate_up[e].to(torch.float32) @ xf[t]
+                a = (gu[:ff] / (1 + torch.exp(-gu[:ff])) * gu[ff:]).to(x.dtype).to(torch.float32)
+                out[t] += weights[t, j] * (w_down[e].to(torch.float32) @ a)
+        if shared is not None:
+            out = out + shared_gate[:, None] * shared.to(torch.float32)
+        return out.to(x.dtype)
+
     def add_rmsnorm(self, resid, delta, weight, eps, out_dtype, rows=None, num_rows=None, lazy=False):
         if rows is None:
             if delta is not None:

@@ -300,10 +300,12 @@ def run_replay(argv: List[str], prog: str = "model_main --replay") -> int:
     from .engine.replay import Replayer
     from .engine.runner import ModelRunner
     args.quantization = "none"
-    model = _load(args, None)
+    # no request grows beyond what all live requests may hold together (a design may set no limit of its own)
+    longest = (max(1, args.max_tokens) + 63) // 64 * 64
+    model = _load(args, longest)
     cfg = model.spec.architecture
     pages = max(1, (args.max_tokens + args.page_size - 1) // args.page_size)
-    step_tokens = args.max_step_tokens or min(max(8192, args.max_live * model.spec.max_positions), 1 << 18)
+    step_tokens = args.max_step_tokens or min(max(8192, args.max_live * min(longest, model.spec.max_positions)), 1 << 18)
     runner = ModelRunner(model, model.env, page_size=args.page_size, num_pages=pages,
                          max_requests=args.max_live, max_batch_tokens=step_tokens)
     print(f"[trace_run] ready: {cfg}, {args.dtype}, {pages} pages of {args.page_size}, "

@@ -1,0 +1,293 @@
+// The gated delta rule: a recurrent mixer with a matrix of state a head.
+//
+// Per row t of a sequence (G key heads of size dk, H value heads of size dv, value head h reads key
+// head h / (H / G)), from the raw projections q, k, v [T, channels]:
+//
+//   prepare:     c  = silu(causal convolution over time, per channel, `taps` taps, zeros before position 0)
+//                q' = unit(c_q) / sqrt(dk),  k' = unit(c_k),  unit(x) = x / sqrt(sum(x^2) + 1e-6),  v' = c_v
+//                beta = sigmoid(b),  decay = exp(-exp(A_log) * softplus(a + dt_bias))
+//   recurrence:  S <- decay S;  u = beta (v' - S^T k');  S <- S + k' u^T;  o = S^T q'
+//   gated norm:  y = o / sqrt(mean(o^2) + eps) * w * silu(gate)         per head, over dv
+//
+// S is float32 [dk, dv] a head and lives in a slot of per-request state, as do the last taps - 1 raw
+// rows that the convolution reads.  A sequence that starts at position 0 has no history: its slot is
+// not read.  Everything after the projections is float32.
+//
+// The recurrence walks a sequence's rows one after the other.  Columns of S are independent, so a
+// column belongs to 8 neighbouring lanes, each holding every 8th of its dk elements in registers; the
+// two dot products of a row (k'.S and q'.S, both with the old S, since
+// o = decay (q'.S_old) + (q'.k') u) are reduced over those lanes together.
+#include "common.h"
+
+__device__ __forceinline__ float silu_f(float z) { return z / (1.0f + expf(-z)); }
+
+// ---------------------------------------------------------------------------------------------
+// prepare: one workgroup a row
+// ---------------------------------------------------------------------------------------------
+template <typename T>
+__global__ void delta_prepare_kernel(const T* __restrict__ proj, int ld, const float* __restrict__ conv_w,
+                                     const T* __restrict__ kept, const float* __restrict__ ba,
+                                     const float* __restrict__ a_log, const float* __restrict__ dt_bias,
+                                     const int* __restrict__ positions, const int* __restrict__ seq_of_row,
+                                     const int* __restrict__ row_start, const int* __restrict__ slots,
+                                     float* __restrict__ qn, float* __restrict__ kn, float* __restrict__ vc,
+                                     float* __restrict__ beta, float* __restrict__ decay, float* __restrict__ qk,
+                                     int H, int G, int dk, int dv, int taps) {
+    extern __shared__ float buf[];                 // the row's channels after convolution and silu
+    const int r = blockIdx.x;
+    const int seq = seq_of_row[r], pos = positions[r];
+    const int in_step = r - row_start[seq];        // rows of this sequence that stand before r in the step
+    const int slot = slots[seq];
+    const int qd = G * dk, C = 2 * qd + H * dv;
+    const T* mine = kept ? kept + (size_t)slot * (taps - 1) * C : nullptr;
+    for (int c = threadIdx.x; c < C; c += blockDim.x) {
+        float acc = 0.f;
+        for (int j = 0; j < taps; ++j) {
+            const int back = taps - 1 - j;          // the tap's row lies this many positions before r
+            if (back > pos) continue;               // before the sequence's first position: zero
+            float x;
+            if (back <= in_step) x = to_f32(proj[(size_t)(r - back) * ld + c]);
+            else x = to_f32(mine[(size_t)(taps - 1 + in_step - back) * C + c]);
+            acc = fmaf(conv_w[(size_t)j * C + c], x, acc);
+        }
+        buf[c] = silu_f(acc);
+    }
+    __syncthreads();
+    const int lane = threadIdx.x % TLI_WAVE, wave = threadIdx.x / TLI_WAVE, waves = blockDim.x / TLI_WAVE;
+    // unit vectors: the 2 G heads of q and k, a wave each in turn
+    for (int v = wave; v < 2 * G; v += waves) {
+        float* x = buf + (size_t)v * dk;
+        float ss = 0.f;
+        for (int i = lane; i < dk; i += TLI_WAVE) ss += x[i] * x[i];
+        ss = wave_sum(ss);
+        float scale = 1.0f / sqrtf(ss + 1e-6f);
+        if (v < G) scale *= 1.0f / sqrtf((float)dk);
+        float* out = (v < G ? qn : kn) + (size_t)r * qd + (size_t)(v < G ? v : v - G) * dk;
+        for (int i = lane; i < dk; i += TLI_WAVE) {
+            const float y = x[i] * scale;
+            x[i] = y;
+            out[i] = y;
+        }
+    }
+    for (int i = threadIdx.x; i < H * dv; i += blockDim.x) vc[(size_t)r * H * dv + i] = buf[2 * qd + i];
+    if (threadIdx.x < H) {
+        const int h = threadIdx.x;
+        const float b = ba[(size_t)r * 2 * H + h], a = ba[(size_t)r * 2 * H + H + h] + dt_bias[h];
+        beta[(size_t)r * H + h] = 1.0f / (1.0f + expf(-b));
+        const float sp = fmaxf(a, 0.f) + log1pf(expf(-fabsf(a)));
+        decay[(size_t)r * H + h] = expf(-expf(a_log[h]) * sp);
+    }
+    __syncthreads();
+    for (int g = wave; g < G; g += waves) {
+        float d = 0.f;
+        for (int i = lane; i < dk; i += TLI_WAVE) d = fmaf(buf[(size_t)g * dk + i], buf[(size_t)(G + g) * dk + i], d);
+        d = wave_sum(d);
+        if (lane == 0) qk[(size_t)r * G + g] = d;
+    }
+}
+
+// The last taps - 1 raw rows of every sequence become its kept rows (oldest first).  Row j of the
+// new kept rows is row n - (taps - 1) + j of the step's n rows, or, where that is negative, kept row
+// n + j of before (zero for a sequence with no history): always a row further on than the one
+// written, so the rows are moved in ascending order in place.
+template <typename T>
+__global__ void delta_conv_keep_kernel(const T* __restrict__ proj, int ld, T* __restrict__ kept,
+                                       const int* __restrict__ row_start, const int* __restrict__ seq_start,
+                                       const int* __restrict__ slots, int C, int taps) {
+    const int seq = blockIdx.y;
+    const int c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= C) return;
+    const int r0 = row_start[seq], n = row_start[seq + 1] - r0;
+    const bool fresh = seq_start[seq] == 0;
+    T* mine = kept + (size_t)slots[seq] * (taps - 1) * C;
+    for (int j = 0; j < taps - 1; ++j) {
+        const int row = n - (taps - 1) + j;
+        T x;
+        if (row >= 0) x = proj[(size_t)(r0 + row) * ld + c];
+        else if (fresh) from_f32(&x, 0.f);
+        else x = mine[(size_t)(n + j) * C + c];
+        mine[(size_t)j * C + c] = x;
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// recurrence
+// ---------------------------------------------------------------------------------------------
+#define DELTA_LANES 8          // lanes that share a column of S
+#define DELTA_COLS 32          // columns a workgroup of 256 threads walks
+
+template <int RPT>             // elements of a column a lane holds: dk <= 8 * RPT
+__global__ __launch_bounds__(256) void delta_recurrence_kernel(
+    const float* __restrict__ qn, const float* __restrict__ kn, const float* __restrict__ vc,
+    const float* __restrict__ beta, const float* __restrict__ decay, const float* __restrict__ qk,
+    float* __restrict__ state, float* __restrict__ out, const int* __restrict__ row_start,
+    const int* __restrict__ seq_start, const int* __restrict__ slots, int H, int G, int dk, int dv) {
+    const int seq = blockIdx.z, head = blockIdx.y;
+    const int part = threadIdx.x % DELTA_LANES;
+    const int col_raw = blockIdx.x * DELTA_COLS + threadIdx.x / DELTA_LANES;
+    const bool live = col_raw < dv;
+    const int col = live ? col_raw : dv - 1;
+    const int kvh = head / (H / G);
+    const int r0 = row_start[seq], r1 = row_start[seq + 1];
+    const bool fresh = seq_start[seq] == 0;
+    float* mine = state + ((size_t)slots[seq] * H + head) * dk * dv;
+    float S[RPT];
+#pragma unroll
+    for (int r = 0; r < RPT; ++r) {
+        const int i = part + DELTA_LANES * r;
+        S[r] = (!fresh && i < dk) ? mine[(size_t)i * dv + col] : 0.f;
+    }
+    const size_t qd = (size_t)G * dk, vd = (size_t)H * dv;
+    float k[RPT], q[RPT], kx[RPT], qx[RPT];
+    float v = 0.f, b = 0.f, g = 0.f, c = 0.f;
+    // the row after the current one is asked for while the current one is worked on
+    auto load = [&](int t, float (&kk)[RPT], float (&qq)[RPT], float& vv, float& bb, float& gg, float& cc) {
+        const float* kp = kn + (size_t)t * qd + (size_t)kvh * dk;
+        const float* qp = qn + (size_t)t * qd + (size_t)kvh * dk;
+#pragma unroll
+        for (int r = 0; r < RPT; ++r) {
+            const int i = part + DELTA_LANES * r;
+            kk[r] = i < dk ? kp[i] : 0.f;
+            qq[r] = i < dk ? qp[i] : 0.f;
+        }
+        vv = vc[(size_t)t * vd + (size_t)head * dv + col];
+        bb = beta[(size_t)t * H + head];
+        gg = decay[(size_t)t * H + head];
+        cc = qk[(size_t)t * G + kvh];
+    };
+    if (r0 < r1) load(r0, kx, qx, v, b, g, c);
+    for (int t = r0; t < r1; ++t) {
+        const float v0 = v, b0 = b, g0 = g, c0 = c;
+#pragma unroll
+        for (int r = 0; r < RPT; ++r) { k[r] = kx[r]; q[r] = qx[r]; }
+        if (t + 1 < r1) load(t + 1, kx, qx, v, b, g, c);
+        float d1 = 0.f, d2 = 0.f;
+#pragma unroll
+        for (int r = 0; r < RPT; ++r) {
+            d1 = fmaf(k[r], S[r], d1);
+            d2 = fmaf(q[r], S[r], d2);
+        }
+#pragma unroll
+        for (int off = 1; off < DELTA_LANES; off <<= 1) {
+            d1 += __shfl_xor(d1, off, TLI_WAVE);
+            d2 += __shfl_xor(d2, off, TLI_WAVE);
+        }
+        const float u = b0 * (v0 - g0 * d1);
+#pragma unroll
+        for (int r = 0; r < RPT; ++r) S[r] = fmaf(k[r], u, g0 * S[r]);
+        if (part == 0 && live) out[(size_t)t * vd + (size_t)head * dv + col] = fmaf(c0, u, g0 * d2);
+    }
+    if (live) {
+#pragma unroll
+        for (int r = 0; r < RPT; ++r) {
+            const int i = part + DELTA_LANES * r;
+            if (i < dk) mine[(size_t)i * dv + col] = S[r];
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// gated norm of the heads' outputs: one wave a (row, head)
+// ---------------------------------------------------------------------------------------------
+template <typename T>
+__global__ void gated_rmsnorm_kernel(const float* __restrict__ o, const T* __restrict__ gate, int gate_ld,
+                                     const float* __restrict__ weight, T* __restrict__ out, int H, int dv, float eps,
+                                     long long pairs) {
+    const long long p = (long long)blockIdx.x * (blockDim.x / TLI_WAVE) + threadIdx.x / TLI_WAVE;
+    if (p >= pairs) return;
+    const int lane = threadIdx.x % TLI_WAVE;
+    const long long row = p / H;
+    const int h = (int)(p - row * H);
+    const float* x = o + (size_t)p * dv;
+    const T* gt = gate + (size_t)row * gate_ld + (size_t)h * dv;
+    float ss = 0.f;
+    for (int i = lane; i < dv; i += TLI_WAVE) ss += x[i] * x[i];
+    ss = wave_sum(ss);
+    const float scale = 1.0f / sqrtf(ss / (float)dv + eps);
+    T* y = out + (size_t)p * dv;
+    for (int i = lane; i < dv; i += TLI_WAVE) from_f32(y + i, x[i] * scale * weight[i] * silu_f(to_f32(gt[i])));
+}
+
+// ---------------------------------------------------------------------------------------------
+// C ABI
+// ---------------------------------------------------------------------------------------------
+#define DELTA_MAX_DK 256
+
+// proj: [T, ld] raw projections, channels q (G dk), k (G dk), v (H dv) first; conv_w: float32
+// [taps, channels], oldest tap first; kept: [slots, taps - 1, channels] or null for one tap;
+// ba: float32 [T, 2 H], b then a.  Outputs are float32: qn, kn [T, G dk], vc [T, H dv], beta, decay
+// [T, H], qk [T, G].  `keep`: also move the kept rows on (after every row was read).
+extern "C" int tli_delta_prepare(const void* proj, int ld, const float* conv_w, void* kept, const float* ba,
+                                 const float* a_log, const float* dt_bias, const int* positions,
+                                 const int* seq_of_row, const int* row_start, const int* seq_start, const int* slots,
+                                 float* qn, float* kn, float* vc, float* beta, float* decay, float* qk, int T,
+                                 int seqs, int H, int G, int dk, int dv, int taps, int dtype, void* stream) {
+    if (T <= 0) return 0;
+    if (H <= 0 || G <= 0 || H % G || dk <= 0 || dv <= 0 || taps <= 0)
+        return tli_fail("delta_prepare: bad sizes (heads %d, key heads %d, dk %d, dv %d, taps %d)", H, G, dk, dv, taps);
+    const int C = 2 * G * dk + H * dv;
+    if (ld < C) return tli_fail("delta_prepare: rows of %d hold fewer than the %d channels", ld, C);
+    if (taps > 1 && !kept) return tli_fail("delta_prepare: %d taps need the sequences' kept rows", taps);
+    if (H > 256) return tli_fail("delta_prepare: at most 256 heads, got %d", H);
+    const size_t lds = (size_t)C * sizeof(float);
+    if (lds > 64 * 1024) return tli_fail("delta_prepare: %d channels do not fit the workgroup's memory", C);
+    hipStream_t s = (hipStream_t)stream;
+    if (dtype == TLI_F32) {
+        hipLaunchKernelGGL((delta_prepare_kernel<float>), dim3(T), dim3(256), lds, s, (const float*)proj, ld, conv_w,
+                           (const float*)kept, ba, a_log, dt_bias, positions, seq_of_row, row_start, slots, qn, kn, vc,
+                           beta, decay, qk, H, G, dk, dv, taps);
+        if (taps > 1)
+            hipLaunchKernelGGL((delta_conv_keep_kernel<float>), dim3((C + 255) / 256, seqs), dim3(256), 0, s,
+                               (const float*)proj, ld, (float*)kept, row_start, seq_start, slots, C, taps);
+    } else if (dtype == TLI_BF16) {
+        hipLaunchKernelGGL((delta_prepare_kernel<bf16_t>), dim3(T), dim3(256), lds, s, (const bf16_t*)proj, ld, conv_w,
+                           (const bf16_t*)kept, ba, a_log, dt_bias, positions, seq_of_row, row_start, slots, qn, kn,
+                           vc, beta, decay, qk, H, G, dk, dv, taps);
+        if (taps > 1)
+            hipLaunchKernelGGL((delta_conv_keep_kernel<bf16_t>), dim3((C + 255) / 256, seqs), dim3(256), 0, s,
+                               (const bf16_t*)proj, ld, (bf16_t*)kept, row_start, seq_start, slots, C, taps);
+    } else {
+        return tli_fail("delta_prepare: unknown dtype %d", dtype);
+    }
+    return tli_check_launch("delta_prepare");
+}
+
+extern "C" int tli_delta_recurrence(const float* qn, const float* kn, const float* vc, const float* beta,
+                                    const float* decay, const float* qk, float* state, float* out,
+                                    const int* row_start, const int* seq_start, const int* slots, int seqs, int H,
+                                    int G, int dk, int dv, void* stream) {
+    if (seqs <= 0) return 0;
+    if (H <= 0 || G <= 0 || H % G || dk <= 0 || dv <= 0 || dk > DELTA_MAX_DK)
+        return tli_fail("delta_recurrence: bad sizes (heads %d, key heads %d, dk %d (at most %d), dv %d)", H, G, dk,
+                        DELTA_MAX_DK, dv);
+    if (H > 65535 || seqs > 65535) return tli_fail("delta_recurrence: too many heads or sequences for one launch");
+    hipStream_t s = (hipStream_t)stream;
+    const dim3 grid((dv + DELTA_COLS - 1) / DELTA_COLS, H, seqs);
+#define TLI_DELTA(RPT) hipLaunchKernelGGL((delta_recurrence_kernel<RPT>), grid, dim3(256), 0, s, qn, kn, vc, beta, \
+                                          decay, qk, state, out, row_start, seq_start, slots, H, G, dk, dv)
+    if (dk <= 16) TLI_DELTA(2);
+    else if (dk <= 32) TLI_DELTA(4);
+    else if (dk <= 64) TLI_DELTA(8);
+    else if (dk <= 128) TLI_DELTA(16);
+    else TLI_DELTA(32);
+#undef TLI_DELTA
+    return tli_check_launch("delta_recurrence");
+}
+
+extern "C" int tli_gated_rmsnorm(const float* o, const void* gate, int gate_ld, const float* weight, void* out,
+                                 int T, int H, int dv, float eps, int dtype, void* stream) {
+    if (T <= 0) return 0;
+    if (H <= 0 || dv <= 0 || gate_ld < H * dv) return tli_fail("gated_rmsnorm: bad sizes");
+    hipStream_t s = (hipStream_t)stream;
+    const long long pairs = (long long)T * H;
+    const int blocks = (int)((pairs + 3) / 4);
+    if (dtype == TLI_F32)
+        hipLaunchKernelGGL((gated_rmsnorm_kernel<float>), dim3(blocks), dim3(256), 0, s, o, (const float*)gate, gate_ld,
+                           weight, (float*)out, H, dv, eps, pairs);
+    else if (dtype == TLI_BF16)
+        hipLaunchKernelGGL((gated_rmsnorm_kernel<bf16_t>), dim3(blocks), dim3(256), 0, s, o, (const bf16_t*)gate,
+                           gate_ld, weight, (bf16_t*)out, H, dv, eps, pairs);
+    else
+        return tli_fail("gated_rmsnorm: unknown dtype %d", dtype);
+    return tli_check_launch("gated_rmsnorm");
+}

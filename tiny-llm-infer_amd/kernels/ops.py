@@ -103,6 +103,12 @@ def load_library():
         "tli_conv_heads": [P, P, P, P, P, P, P, P, P, P, I, I, P, I, I, I, I, I, I, I, I, I, P],
         "tli_attention_biased_plain": [P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, P, P, P, I, I, I, P],
         "tli_attention_biased_mfma_bf16": [P, P, P, P, P, P, I, I, I, P, I, I, I, I, I, I, F, P, P, P, I, I, I, P],
+        "tli_add_layernorm": [P, P, P, P, P, P, P, P, I, I, I, F, I, P],
+        "tli_delta_prepare": [P, I, P, P, P, P, P, P, P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, P],
+        "tli_delta_recurrence": [P, P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, P],
+        "tli_gated_rmsnorm": [P, P, I, P, P, I, I, I, F, I, P],
+        "tli_moe_route": [P, I, P, P, P, I, I, I, I, I, F, I, P],
+        "tli_moe_experts": [P, P, P, P, P, P, P, P, P, I, I, I, I, I, P],
         "tli_sample": [P, I, I, P, P, P, P, P, P],
         "tli_sample_scratch_bytes": [I],
         "tli_random_normal": [P, ctypes.c_longlong, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint32, P, F, F, I, P],
@@ -1026,6 +1032,153 @@ class HipOps:
                    step.positions.data_ptr(), step.seq_of_row.data_ptr(), g.tables.data_ptr(), g.table_width,
                    g.page_size, kc.shape[0], T, heads, kv_heads, head_dim, float(scale), _ptr(temp), _ptr(r1), _ptr(r2),
                    kind, size, _dtype_code(qk.dtype), self._stream())
+        return out
+
+    # ---- layer norm ------------------------------------------------------------------------------
+    def add_layernorm(self, resid, deltas, weights, eps, out_dtype, rows=None, num_rows=None):
+        """``resid`` (float32 [T, n]) takes the sum of ``deltas`` (none, one or two tensors [T, n] of
+        ``out_dtype``: what the parts before still owe it); returns the layer norm (no bias) of its rows
+        once for every weight vector of ``weights`` (one or two: norms of the same rows share their mean
+        and variance).  With ``rows`` only those rows are computed and ``resid`` stays as it is."""
+        total, n = resid.shape
+        self._want(resid, "residual", torch.float32)
+        deltas = tuple(deltas)
+        if len(deltas) > 2 or not 1 <= len(weights) <= 2:
+            raise KernelError("add_layernorm takes at most two deltas and one or two weight vectors")
+        for d in deltas:
+            self._want(d, "residual delta", out_dtype, (total, n))
+        for w in weights:
+            self._want(w, "norm weight", torch.float32, (n,))
+        out_rows = total
+        if rows is not None:
+            self._want(rows, "row list", torch.int32)
+            out_rows = rows.numel() if num_rows is None else num_rows
+            if rows.numel() < out_rows:
+                raise KernelError("row list is shorter than the rows asked for")
+        outs = [torch.empty((out_rows, n), dtype=out_dtype, device=self.device) for _ in weights]
+        d1 = deltas[0] if deltas else None
+        d2 = deltas[1] if len(deltas) > 1 else None
+        self._call(self.lib.tli_add_layernorm, resid.data_ptr(), _ptr(d1), _ptr(d2), weights[0].data_ptr(),
+                   _ptr(weights[1]) if len(weights) > 1 else None, outs[0].data_ptr(),
+                   outs[1].data_ptr() if len(weights) > 1 else None, _ptr(rows), out_rows, total, n, float(eps),
+                   _dtype_code(out_dtype), self._stream())
+        return outs
+
+    # ---- the gated delta rule ----------------------------------------------------------------------
+    MAX_DELTA_KEY_DIM = 256
+
+    def check_delta_sizes(self, heads: int, kv_heads: int, dk: int, dv: int, taps: int) -> None:
+        if heads <= 0 or kv_heads <= 0 or heads % kv_heads or heads > 256:
+            raise KernelError(f"{heads} heads (at most 256) cannot be grouped over {kv_heads} key heads")
+        if not 1 <= dk <= self.MAX_DELTA_KEY_DIM or dv < 1:
+            raise KernelError(f"a state of {dk} x {dv} a head is not supported: key heads of 1 to {self.MAX_DELTA_KEY_DIM}")
+        if not 1 <= taps <= self.MAX_CONV_TAPS:
+            raise KernelError(f"a convolution of {taps} taps is not supported: 1 to {self.MAX_CONV_TAPS}")
+        if (2 * kv_heads * dk + heads * dv) * 4 > 64 * 1024:
+            raise KernelError("the channels of q, k and v of a row do not fit a workgroup's memory")
+
+    def delta_rule(self, proj, gates, conv, a_log, dt_bias, kept, state, step, heads, kv_heads, dk, dv, taps):
+        """From the raw projections ``proj`` [T, >= channels] (q, k, v first) and ``gates`` (float32 [T, 2 H]:
+        b, then a) to the heads' outputs of the recurrence, float32 [T, H dv].  ``conv``: float32 [taps,
+        channels], oldest tap first; ``kept`` [slots, taps - 1, channels] and ``state`` (float32 [slots, H,
+        dk, dv]) are the sequences' state, read (unless a sequence starts at position 0) and replaced."""
+        T = step.num_rows
+        self.check_delta_sizes(heads, kv_heads, dk, dv, taps)
+        qd, vd = kv_heads * dk, heads * dv
+        C = 2 * qd + vd
+        if proj.dim() != 2 or proj.shape[0] != T or proj.shape[1] < C:
+            raise KernelError(f"the projections have shape {tuple(proj.shape)}, expected [{T}, >= {C}]")
+        self._want(proj, "projections")
+        self._want(gates, "b and a", torch.float32, (T, 2 * heads))
+        self._want(conv, "convolution weights", torch.float32, (taps, C))
+        self._want(a_log, "A_log", torch.float32, (heads,))
+        self._want(dt_bias, "dt_bias", torch.float32, (heads,))
+        self._want(state, "recurrent state", torch.float32, (state.shape[0], heads, dk, dv))
+        slots = state.shape[0]
+        if taps > 1:
+            if kept is None:
+                raise KernelError("the convolution needs the sequences' kept rows")
+            self._want(kept, "kept rows of the convolution", proj.dtype, (slots, taps - 1, C))
+        if max(step.h_slots, default=0) >= slots:
+            raise KernelError("a sequence's slot lies outside the state")
+        f32 = dict(dtype=torch.float32, device=self.device)
+        qn, kn = torch.empty((T, qd), **f32), torch.empty((T, qd), **f32)
+        vc, out = torch.empty((T, vd), **f32), torch.empty((T, vd), **f32)
+        beta, decay, qk = torch.empty((T, heads), **f32), torch.empty((T, heads), **f32), torch.empty((T, kv_heads), **f32)
+        self._call(self.lib.tli_delta_prepare, proj.data_ptr(), proj.shape[1], conv.data_ptr(), _ptr(kept), gates.data_ptr(),
+                   a_log.data_ptr(), dt_bias.data_ptr(), step.positions.data_ptr(), step.seq_of_row.data_ptr(),
+                   step.row_start.data_ptr(), step.seq_start.data_ptr(), step.slots.data_ptr(), qn.data_ptr(),
+                   kn.data_ptr(), vc.data_ptr(), beta.data_ptr(), decay.data_ptr(), qk.data_ptr(), T, step.num_seqs,
+                   heads, kv_heads, dk, dv, taps, _dtype_code(proj.dtype), self._stream())
+        self._call(self.lib.tli_delta_recurrence, qn.data_ptr(), kn.data_ptr(), vc.data_ptr(), beta.data_ptr(),
+                   decay.data_ptr(), qk.data_ptr(), state.data_ptr(), out.data_ptr(), step.row_start.data_ptr(),
+                   step.seq_start.data_ptr(), step.slots.data_ptr(), step.num_seqs, heads, kv_heads, dk, dv, self._stream())
+        return out
+
+    def gated_rmsnorm(self, o, proj, gate_at, weight, eps, heads, dv, out_dtype):
+        """y = o / sqrt(mean(o^2) + eps) * weight * silu(gate) per head; ``o`` float32 [T, H dv], the gate
+        is columns ``gate_at`` .. ``gate_at + H dv`` of ``proj``."""
+        T = o.shape[0]
+        self._want(o, "heads' outputs", torch.float32, (T, heads * dv))
+        self._want(proj, "projections", out_dtype)
+        if proj.shape[0] != T or proj.shape[1] < gate_at + heads * dv:
+            raise KernelError("the gate lies outside the projections")
+        self._want(weight, "norm weight", torch.float32, (dv,))
+        out = torch.empty((T, heads * dv), dtype=out_dtype, device=self.device)
+        self._call(self.lib.tli_gated_rmsnorm, o.data_ptr(), proj.data_ptr() + gate_at * proj.element_size(), proj.shape[1],
+                   weight.data_ptr(), out.data_ptr(), T, heads, dv, float(eps), _dtype_code(out_dtype), self._stream())
+        return out
+
+    # ---- routed experts ---------------------------------------------------------------------------------
+    MAX_EXPERTS_TOP = 32
+
+    def check_expert_sizes(self, experts, top, groups, keep, hidden, inter) -> None:
+        if not 1 <= top <= min(experts, self.MAX_EXPERTS_TOP) or experts > 2048:
+            raise KernelError(f"{top} of {experts} experts a row: at most {self.MAX_EXPERTS_TOP} of at most 2048")
+        if not 1 <= groups <= 64 or experts % groups or not 1 <= keep <= groups or keep * (experts // groups) < top:
+            raise KernelError(f"{experts} experts in {groups} groups (at most 64), {keep} kept: cannot give {top}")
+        if hidden * 4 > 64 * 1024 or top * inter * 4 > 64 * 1024:
+            raise KernelError("a row, or the hidden units of a row's experts, do not fit a workgroup's memory")
+
+    def pack_experts(self, w_gate_up, w_down):
+        """Whatever other layout of the experts' matrices the kernels for many rows want (none yet)."""
+        return None
+
+    def route_experts(self, z, experts, top, groups, keep, scale, has_shared):
+        """From router logits ``z`` (float32 [T, E (+ 1)]) to the chosen experts (int32 [T, top]), their
+        weights (float32 [T, top]) and, if the last column is a shared expert's gate, its sigmoid [T]."""
+        T = z.shape[0]
+        self._want(z, "router logits", torch.float32, (T, experts + (1 if has_shared else 0)))
+        ids = torch.empty((T, top), dtype=torch.int32, device=self.device)
+        weights = torch.empty((T, top), dtype=torch.float32, device=self.device)
+        gate = torch.empty((T,), dtype=torch.float32, device=self.device) if has_shared else None
+        self._call(self.lib.tli_moe_route, z.data_ptr(), z.shape[1], ids.data_ptr(), weights.data_ptr(), _ptr(gate), T,
+                   experts, top, groups, keep, float(scale), 1 if has_shared else 0, self._stream())
+        return ids, weights, gate
+
+    def apply_experts(self, x, ids, weights, w_gate_up, w_down, packed, shared, shared_gate):
+        """sum_j weights[t, j] * expert ids[t, j] (x[t])  (+ shared_gate[t] * shared[t]);  ``w_gate_up``
+        [E, 2 ff, n] (an expert's gate rows, then its up rows), ``w_down`` [E, n, ff]."""
+        T, n = x.shape
+        E, two_ff, _ = w_gate_up.shape
+        ff, top = two_ff // 2, ids.shape[1]
+        self._want(x, "expert input")
+        self._want(w_gate_up, "experts' gate and up matrices", x.dtype, (E, 2 * ff, n))
+        self._want(w_down, "experts' down matrices", x.dtype, (E, n, ff))
+        self._want(ids, "chosen experts", torch.int32, (T, top))
+        self._want(weights, "experts' weights", torch.float32, (T, top))
+        if shared is not None:
+            self._want(shared, "shared expert's output", x.dtype, (T, n))
+            self._want(shared_gate, "shared expert's gate", torch.float32, (T,))
+        out = torch.empty((T, n), dtype=x.dtype, device=self.device)
+        hid = torch.empty((T * top, ff), dtype=x.dtype, device=self.device)
+        for t0 in range(0, T, 32768):
+            t1 = min(T, t0 + 32768)
+            self._call(self.lib.tli_moe_experts, x[t0:t1].data_ptr(), ids[t0:t1].data_ptr(), weights[t0:t1].data_ptr(),
+                       w_gate_up.data_ptr(), w_down.data_ptr(), hid[t0 * top:].data_ptr(),
+                       None if shared is None else shared[t0:t1].data_ptr(),
+                       None if shared is None else shared_gate[t0:t1].data_ptr(), out[t0:t1].data_ptr(), t1 - t0, top, n, ff,
+                       _dtype_code(x.dtype), self._stream())
         return out
 
     def sample(self, logits: torch.Tensor, temperatures: Optional[torch.Tensor] = None,

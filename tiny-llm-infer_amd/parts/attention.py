@@ -10,6 +10,18 @@ p-window+1..p for a windowed layer, softmax, weighted sum of values -> output
 projection.  v is neither normed nor rotated.  Every row reads its keys from
 the cache, the step's own rows included, so a portion of a prompt and a single
 decoded token are the same case.
+
+``norm_after_rotation``: the design norms q and k after it has turned them.  A rotation
+leaves the sum of squares of a pair as it is, so for a norm whose weights are equal within
+every turned pair (a norm without weights is one) the two orders give the same numbers, and
+the kernels' order serves.  Any other norm is refused with that flag.
+
+``value_dim``: value heads of another size than the query/key heads.  The kernels know one
+head size P, so every head is laid out in P = max(head_dim, value_dim) elements (rounded up to
+a multiple of 16), the rows of the projections that do not exist being zero (and the
+columns of the output projection likewise).  Zeros change no score and no sum; the RMS norm
+of a head of d elements held in P is the norm over P with weights w sqrt(d / P) and
+eps d / P, which is what the kernels are given.
 """
 from __future__ import annotations
 
@@ -34,23 +46,27 @@ class PagedAttention(Mixer):
         self.kv_heads = int(p["num_kv_heads"])
         self.head_dim = int(p["head_dim"])
         self.scale = float(p["scale"])
+        self.value_dim = int(p.get("value_dim") or self.head_dim)
+        self.norm_after_rotation = bool(p.get("norm_after_rotation", False))
+        # the one head size that the kernels and the cache see
+        self.padded = self.head_dim if self.value_dim == self.head_dim else (max(self.head_dim, self.value_dim) + 15) // 16 * 16
         self.window = None if p.get("window") is None else int(p["window"])
         if self.heads % self.kv_heads:
             raise ValueError("num_heads must be a multiple of num_kv_heads")
         if self.window is not None and self.window <= 0:
             raise ValueError("window must be positive")
-        self.q_dim = self.heads * self.head_dim
-        self.kv_dim = self.kv_heads * self.head_dim
+        self.q_dim = self.heads * self.padded
+        self.kv_dim = self.kv_heads * self.padded
         self.position = build_part("position", spec.parts["position"]) if "position" in spec.parts else None
         self.q_norm = build_part("norm", spec.parts["q_norm"]) if "q_norm" in spec.parts else None
         self.k_norm = build_part("norm", spec.parts["k_norm"]) if "k_norm" in spec.parts else None
 
     def tensors(self) -> List[TensorDecl]:
         n = self.spec.names
-        out = [TensorDecl(n["q"], (self.q_dim, self.hidden)),
-               TensorDecl(n["k"], (self.kv_dim, self.hidden)),
-               TensorDecl(n["v"], (self.kv_dim, self.hidden)),
-               TensorDecl(n["o"], (self.hidden, self.q_dim))]
+        out = [TensorDecl(n["q"], (self.heads * self.head_dim, self.hidden)),
+               TensorDecl(n["k"], (self.kv_heads * self.head_dim, self.hidden)),
+               TensorDecl(n["v"], (self.kv_heads * self.value_dim, self.hidden)),
+               TensorDecl(n["o"], (self.hidden, self.heads * self.value_dim))]
         for part in (self.q_norm, self.k_norm, self.position):
             if part is not None:
                 out += part.tensors()
@@ -62,7 +78,7 @@ class PagedAttention(Mixer):
         for part in (self.q_norm, self.k_norm, self.position):
             if part is not None:
                 part.load(weights, env)
-        env.ops.check_attention_sizes(self.heads, self.kv_heads, self.head_dim)
+        env.ops.check_attention_sizes(self.heads, self.kv_heads, self.padded)
         # The kernels turn the pairs (i, i + rotary_dim/2) of a head.  An encoding that pairs
         # neighbours (2i, 2i + 1) is served by the same kernels: a head's scores q.k do not change
         # when q and k are permuted alike, so the rows of the q and k projections (and the weights
@@ -92,19 +108,45 @@ class PagedAttention(Mixer):
                 weight, eps = rms
                 if tuple(weight.shape) != (self.head_dim,):
                     raise ValueError(f"the {role} norm has {tuple(weight.shape)} weights, a head has {self.head_dim} elements")
-                rms = (weight[order.to(weight.device)].contiguous() if order is not None else weight, float(eps))
+                if self.norm_after_rotation and self.rotary is not None:
+                    rd, half = self.rotary[2], self.rotary[2] // 2
+                    pairs = (weight[0:rd:2], weight[1:rd:2]) if order is not None else (weight[:half], weight[half:rd])
+                    if not torch.equal(*pairs):
+                        raise ValueError(f"the {role} norm comes after the rotation and its weights differ within "
+                                         f"a turned pair: the attention kernels norm first")
+                weight = weight[order.to(weight.device)].contiguous() if order is not None else weight
+                if self.padded != self.head_dim:
+                    ratio = self.head_dim / self.padded
+                    wide = torch.zeros(self.padded, dtype=torch.float32, device=weight.device)
+                    wide[:self.head_dim] = weight * ratio ** 0.5
+                    weight, eps = wide, float(eps) * ratio
+                rms = (weight, float(eps))
             self.head_norms.append(rms)
 
-        def heads_in_order(w: torch.Tensor, heads: int) -> torch.Tensor:
-            if order is None:
+        def widened(w: torch.Tensor, heads: int, size: int) -> torch.Tensor:
+            """Heads of ``size`` rows laid out in ``padded`` rows each, zeros behind."""
+            if size == self.padded:
                 return w
-            return w.view(heads, self.head_dim, self.hidden)[:, order.to(w.device)].reshape(heads * self.head_dim, self.hidden)
+            wide = torch.zeros((heads, self.padded, self.hidden), dtype=w.dtype, device=w.device)
+            wide[:, :size] = w.view(heads, size, self.hidden)
+            return wide.view(heads * self.padded, self.hidden)
+
+        def heads_in_order(w: torch.Tensor, heads: int) -> torch.Tensor:
+            if order is not None:
+                w = w.view(heads, self.head_dim, self.hidden)[:, order.to(w.device)].reshape(heads * self.head_dim, self.hidden)
+            return widened(w, heads, self.head_dim)
         self.w_qkv = fuse_rows([heads_in_order(weights[n["q"]], self.heads),
-                                heads_in_order(weights[n["k"]], self.kv_heads), weights[n["v"]]], env)
-        self.w_o = as_matrix(weights[n["o"]], env)
+                                heads_in_order(weights[n["k"]], self.kv_heads),
+                                widened(weights[n["v"]], self.kv_heads, self.value_dim)], env)
+        w_o = weights[n["o"]]
+        if self.value_dim != self.padded:
+            wide = torch.zeros((self.hidden, self.heads, self.padded), dtype=w_o.dtype, device=w_o.device)
+            wide[:, :, :self.value_dim] = w_o.view(self.hidden, self.heads, self.value_dim)
+            w_o = wide.view(self.hidden, self.heads * self.padded)
+        self.w_o = as_matrix(w_o, env)
 
     def cache_need(self) -> Optional[CacheNeed]:
-        return CacheNeed.keys_and_values(self.kv_heads, self.head_dim, self.window)
+        return CacheNeed.keys_and_values(self.kv_heads, self.padded, self.window)
 
     def workspace_elems(self, rows: int) -> int:
         # q, k, v rows (as float32 partial sums at worst), the rotated q, the attention's output
@@ -117,7 +159,7 @@ class PagedAttention(Mixer):
     def forward(self, x: torch.Tensor, step: StepView) -> torch.Tensor:
         ops = self.env.ops
         qkv = ops.linear(x, self.w_qkv, sums_only=True)      # partial sums, if k was split, are the attention's to add
-        o = ops.qkv_attention(qkv, step, step.cache, self.heads, self.kv_heads, self.head_dim,
+        o = ops.qkv_attention(qkv, step, step.cache, self.heads, self.kv_heads, self.padded,
                               self.head_norms[0], self.head_norms[1], self.rotary, self.scale, self.window)
         return ops.linear(o, self.w_o, deferred=True)       # goes to the next norm as the residual delta
 

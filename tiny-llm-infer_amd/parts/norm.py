@@ -1,7 +1,11 @@
 """RMSNorm: y_j = w_j * x_j / sqrt(mean(x^2) + eps), all in float32
-(kernels/src/rmsnorm_kernel_cpu.cpp:27-43).  The weight is a plain multiplier.
+(kernels/src/rmsnorm_kernel_cpu.cpp:27-43).  The weight is a plain multiplier; a
+norm whose spec names no weight has none (all ones).
 The residual stream is float32; the norm adds what the previous part owes the
-residual before it normalises, so the residual sum is never rounded."""
+residual before it normalises, so the residual sum is never rounded.
+
+LayerNorm: y_j = w_j * (x_j - m) / sqrt(mean((x - m)^2) + eps) with m = mean(x), a
+weight and no bias, float32 likewise."""
 from __future__ import annotations
 
 from typing import Dict, List, Optional
@@ -21,16 +25,19 @@ class RMSNorm(Norm):
         super().__init__(spec)
         self.size = int(spec.params["size"])
         self.eps = float(spec.params["eps"])
-        self.weight_name = spec.names["weight"]
+        self.weight_name = spec.names.get("weight")             # None: a norm without weights
         self.weight: Optional[torch.Tensor] = None
 
     def tensors(self) -> List[TensorDecl]:
-        return [TensorDecl(self.weight_name, (self.size,), "ones_normal")]
+        return [TensorDecl(self.weight_name, (self.size,), "ones_normal")] if self.weight_name is not None else []
 
     def load(self, weights: Dict[str, torch.Tensor], env: BuildEnv) -> None:
         super().load(weights, env)
         # vectors are held in float32: exact for 16-bit storage, unchanged for 32-bit
-        self.weight = weights[self.weight_name].to(torch.float32).contiguous()
+        if self.weight_name is None:
+            self.weight = torch.ones(self.size, dtype=torch.float32, device=env.device)
+        else:
+            self.weight = weights[self.weight_name].to(torch.float32).contiguous()
 
     def as_rms(self):
         return self.weight, self.eps
@@ -42,4 +49,33 @@ class RMSNorm(Norm):
                                         rows=rows, num_rows=num_rows, **({"lazy": True} if lazy else {}))
 
 
+class LayerNorm(Norm):
+    replayable = True
+
+    def __init__(self, spec):
+        super().__init__(spec)
+        self.size = int(spec.params["size"])
+        self.eps = float(spec.params["eps"])
+        self.weight_name = spec.names["weight"]
+        self.weight: Optional[torch.Tensor] = None
+
+    def tensors(self) -> List[TensorDecl]:
+        return [TensorDecl(self.weight_name, (self.size,), "ones_normal")]
+
+    def load(self, weights: Dict[str, torch.Tensor], env: BuildEnv) -> None:
+        super().load(weights, env)
+        self.weight = weights[self.weight_name].to(torch.float32).contiguous()
+
+    def as_layer_norm(self):
+        """(weight float32 [size], eps): for an arrangement that norms one row with two such norms
+        in one pass."""
+        return self.weight, self.eps
+
+    def forward(self, resid, delta, rows=None, num_rows=None):
+        deltas = () if delta is None else (delta,)
+        return self.env.ops.add_layernorm(resid, deltas, (self.weight,), self.eps, self.env.dtype,
+                                          rows=rows, num_rows=num_rows)[0]
+
+
 register_part("norm", "rmsnorm", RMSNorm)
+register_part("norm", "layernorm", LayerNorm)
