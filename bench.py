@@ -66,13 +66,14 @@ DESIGN_SIZES = {
 
 
 def compare_designs(args):
-    """Prefill and decode of the Sinepel design beside the Qwen3 dense decoder at equal layer sizes
+    """Prefill and decode of the Sinepel design (or, with --design-names, of others: Kapanex) beside the Qwen3
+    dense decoder at equal layer sizes
     (random bfloat16 weights, 4 layers unless --layers says otherwise), through the step function:
     one prompt of --prefill-tokens in one step, and decode steps of --batch and 64 requests at
     --prompt-len tokens of context.  One JSON line."""
     import torch
 
-    from tiny_llm_infer_amd.config import Qwen3Config, SinepelConfig
+    from tiny_llm_infer_amd.config import KapanexConfig, Qwen3Config, SinepelConfig
     from tiny_llm_infer_amd.engine.loading import random_model
     from tiny_llm_infer_amd.engine.runner import ModelRunner, StepEntry
     import random
@@ -98,7 +99,26 @@ def compare_designs(args):
         qwen = Qwen3Config.from_dict(dict(QWEN3_8B, hidden_size=width, intermediate_size=ff, num_hidden_layers=layers,
                                           num_attention_heads=heads, num_key_value_heads=kv_heads, head_dim=dim,
                                           vocab_size=vocab, max_position_embeddings=context))
-        for design, arch, cfg in (("sinepel", "Sinepel", sinepel), ("qwen3", "Qwen3ForCausalLM", qwen)):
+        # Kapanex: attention (a window of 1,024, half of every head turned) and delta-rule layers in turn, heads
+        # as Qwen3's; 16 experts of a quarter of the feed-forward size in 4 groups of which 2 are kept, 2 chosen,
+        # beside a shared expert of half of it: as many feed-forward weights at work on a token as Qwen3 has
+        moe = {"kind": "moe", "expert": {"ff": ff // 4}, "shared": {"ff": ff // 2},
+               "router": {"experts": 16, "top": 2, "scale": 2.0, "groups": {"count": 4, "keep": 2}}}
+        kapanex = KapanexConfig.from_dict({
+            "architecture": "Kapanex", "vocab": vocab, "width": width, "embedding": {"scale": 1.0}, "norm": {"eps": 1e-5},
+            "max_positions": context,
+            "layers": [{"type": "attention", "mlp": moe,
+                        "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5,
+                                  "mask": {"size": 1024}, "rot": {"dims": dim // 2, "base": 1e6}}} if i % 2 == 0 else
+                       {"type": "delta", "mlp": moe,
+                        "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "conv": 4}}
+                       for i in range(layers)]})
+        known = {"sinepel": ("Sinepel", sinepel), "kapanex": ("Kapanex", kapanex), "qwen3": ("Qwen3ForCausalLM", qwen)}
+        names = [n for n in args.design_names.split(",") if n]
+        if any(n not in known for n in names):
+            print(f"--design-names: known designs are {', '.join(known)}")
+            return 2
+        for design, arch, cfg in ((n,) + known[n] for n in names):
             model = random_model(arch, cfg, args.seed, args.dtype, "cuda:0", context)
             batches = sorted({args.batch, 64})
             pages = (args.prefill_tokens + page - 1) // page + max(batches) * ((args.prompt_len + args.steps + args.warmup + 80) // page + 2)
@@ -173,6 +193,8 @@ def main():
     ap.add_argument("--designs", default=None,
                     help="instead of the default workload: the Sinepel design beside the Qwen3 dense decoder at equal layer "
                          f"sizes, prefill and decode; a list of {','.join(DESIGN_SIZES)} or 'all'")
+    ap.add_argument("--design-names", default="sinepel,qwen3",
+                    help="with --designs: which designs are run at every size (sinepel, kapanex, qwen3)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py runs on one GPU only; --gpus {args.gpus} is not supported (single-GPU engine)")

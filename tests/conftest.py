@@ -28,3 +28,19 @@ def sinepel_folders(tmp_path_factory):
     from sinepel_helpers import SMALL, make_folder
     root = tmp_path_factory.mktemp("sinepel")
     return {name: make_folder(str(root / name), name) for name in SMALL}
+
+
+@pytest.fixture(scope="session")
+def kapanex_folders(tmp_path_factory):
+    """Model folders of the small Kapanex configurations, made once in a temporary folder."""
+    from kapanex_helpers import SMALL, make_folder
+    root = tmp_path_factory.mktemp("kapanex")
+    return {name: make_folder(str(root / name), name) for name in SMALL}
+
+
+@pytest.fixture(scope="session")
+def kapanex_clear_folders(tmp_path_factory):
+    """The same configurations with weights whose routers never have a close call (for comparisons in bfloat16)."""
+    from kapanex_helpers import SMALL, make_folder
+    root = tmp_path_factory.mktemp("kapanex_clear")
+    return {name: make_folder(str(root / name), name, clear_routing=True) for name in SMALL}

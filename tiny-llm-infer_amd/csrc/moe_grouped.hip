@@ -1,0 +1,286 @@
+// Routed experts on the matrix cores (bfloat16): the (row, chosen expert) pairs of a step are sorted
+// by expert, and every expert multiplies its pairs tile by tile, reading its matrices once a tile.
+//
+//   sort:     pairs of one expert get consecutive slots, an expert's run of slots filled up to whole
+//             tiles of RT slots (`order`: slot -> pair or -1, `pos`: pair -> slot, `tile_expert`: tile ->
+//             expert).  How many tiles there are is known on the device only: the products are launched
+//             for the most there can be (pairs / RT + experts) and a workgroup without a tile leaves.
+//   gate/up:  hid[slot, f] = silu(x[row] . Wg_e[f]) * (x[row] . Wu_e[f])          (bfloat16)
+//   down:     part[slot, c] = hid[slot] . Wd_e[c]                                 (float32)
+//   combine:  y[row] = sum_j weight[row, j] part[pos[row, j]]  (+ shared gate * shared), in the order of
+//             the choice: a row's result does not depend on which other rows share its tiles, because the
+//             rows of a tile never meet in a sum.
+//
+// The matrices are read in the tiled layout of the other products (blocks of 16 rows x 128 columns, 4
+// KiB, in the order the operands of v_mfma_f32_16x16x32_bf16 want: a load instruction of a wave takes 1 KiB
+// in a row); rows and columns that do not exist are zeros there.  A is a tile of W (16 outputs), B the
+// rows of x, so a lane ends with 4 consecutive outputs of one row.  A wave takes 16 outputs and all RT
+// rows of its tile; the four waves of a workgroup share the rows of x through the cache.
+#include "common.h"
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4g;
+union Frag {
+    uint4 u;
+    u32x4g w;
+    bf16x8 v;
+};
+
+__device__ __forceinline__ Frag frag_load(const bf16_t* p) {
+    Frag f;
+    f.u = *reinterpret_cast<const uint4*>(p);
+    return f;
+}
+__device__ __forceinline__ Frag frag_load_if(const bf16_t* p, bool ok) {
+    Frag f;
+    f.u = ok ? *reinterpret_cast<const uint4*>(p) : make_uint4(0, 0, 0, 0);
+    return f;
+}
+
+// ---------------------------------------------------------------------------------------------
+// sort: one workgroup
+// ---------------------------------------------------------------------------------------------
+#define SORT_MAX_EXPERTS 2048
+
+__global__ void __launch_bounds__(1024) moe_sort_kernel(const int* __restrict__ ids, int P, int E, int RT,
+                                                         int tiles_max, int* __restrict__ order,
+                                                         int* __restrict__ pos, int* __restrict__ tile_expert,
+                                                         int* __restrict__ num_tiles) {
+    __shared__ int count[SORT_MAX_EXPERTS], start[SORT_MAX_EXPERTS], fill[SORT_MAX_EXPERTS];
+    for (int e = threadIdx.x; e < E; e += blockDim.x) count[e] = fill[e] = 0;
+    __syncthreads();
+    for (int p = threadIdx.x; p < P; p += blockDim.x) {
+        int e = ids[p];
+        if (e < 0 || e >= E) e = 0;                   // (the router gives no such id)
+        atomicAdd(&count[e], 1);
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < E; e += blockDim.x) {
+        int before = 0;                               // tiles of the experts before e
+        for (int i = 0; i < e; ++i) before += (count[i] + RT - 1) / RT;
+        start[e] = before * RT;
+        const int mine = (count[e] + RT - 1) / RT;
+        for (int i = 0; i < mine; ++i) tile_expert[before + i] = e;
+        if (e == E - 1) {
+            *num_tiles = before + mine;
+            for (int i = before + mine; i < tiles_max; ++i) tile_expert[i] = -1;
+        }
+    }
+    for (int s = threadIdx.x; s < tiles_max * RT; s += blockDim.x) order[s] = -1;
+    __syncthreads();
+    for (int p = threadIdx.x; p < P; p += blockDim.x) {
+        int e = ids[p];
+        if (e < 0 || e >= E) e = 0;
+        const int slot = start[e] + atomicAdd(&fill[e], 1);
+        order[slot] = p;
+        pos[p] = slot;
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// gate and up products with the activation
+// ---------------------------------------------------------------------------------------------
+__device__ __forceinline__ float grouped_silu(float z) { return z / (1.0f + expf(-z)); }
+
+template <int RB>            // a tile has 16 RB slots
+__global__ void __launch_bounds__(256) moe_gate_up_kernel(const bf16_t* __restrict__ x, const int* __restrict__ order,
+                                                           const int* __restrict__ tile_expert,
+                                                           const int* __restrict__ num_tiles,
+                                                           const bf16_t* __restrict__ gate_t,
+                                                           const bf16_t* __restrict__ up_t, bf16_t* __restrict__ hid,
+                                                           int top, int D, int ff) {
+    const int tile = blockIdx.y;
+    if (tile >= *num_tiles) return;
+    const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
+    const int r = lane % 16, c = lane / 16;
+    const int nb = blockIdx.x * 4 + wave;             // the wave's block of 16 hidden units
+    const int nblocks = (ff + 15) / 16, kblocks = (D + 127) / 128;
+    if (nb >= nblocks) return;
+    const int e = tile_expert[tile];
+    const size_t block0 = ((size_t)e * nblocks + nb) * kblocks * 2048 + lane * 8;
+    const bf16_t* wg = gate_t + block0;
+    const bf16_t* wu = up_t + block0;
+    const bf16_t* xr[RB];
+    int slot[RB];
+    bool live[RB];
+#pragma unroll
+    for (int b = 0; b < RB; ++b) {
+        slot[b] = (tile * RB + b) * 16 + r;
+        const int p = order[slot[b]];
+        live[b] = p >= 0;
+        xr[b] = x + (size_t)(live[b] ? p / top : 0) * D + c * 32;       // (a slot without a pair reads row 0 and stores nothing)
+    }
+    f32x4 ag[RB], au[RB];
+#pragma unroll
+    for (int b = 0; b < RB; ++b) ag[b] = au[b] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    const int whole = D / 128;
+    for (int kb = 0; kb < whole; ++kb) {
+        Frag fg[4], fu[4], fx[RB][4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            fg[j] = frag_load(wg + (size_t)kb * 2048 + j * 512);
+            fu[j] = frag_load(wu + (size_t)kb * 2048 + j * 512);
+#pragma unroll
+            for (int b = 0; b < RB; ++b) fx[b][j] = frag_load(xr[b] + kb * 128 + j * 8);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int b = 0; b < RB; ++b) {
+                ag[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fg[j].v, fx[b][j].v, ag[b], 0, 0, 0);
+                au[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fu[j].v, fx[b][j].v, au[b], 0, 0, 0);
+            }
+    }
+    if (whole < kblocks) {                            // the last, partial block of k: rows of x end before it does
+        const int kb = whole;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const Frag fg = frag_load(wg + (size_t)kb * 2048 + j * 512);
+            const Frag fu = frag_load(wu + (size_t)kb * 2048 + j * 512);
+            const bool ok = kb * 128 + c * 32 + j * 8 + 8 <= D;
+#pragma unroll
+            for (int b = 0; b < RB; ++b) {
+                const Frag fx = frag_load_if(xr[b] + kb * 128 + j * 8, ok);
+                ag[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fg.v, fx.v, ag[b], 0, 0, 0);
+                au[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fu.v, fx.v, au[b], 0, 0, 0);
+            }
+        }
+    }
+    // the lane holds hidden units nb * 16 + 4 c .. + 4 of the slots 16 b + r
+    const int n0 = nb * 16 + c * 4;
+#pragma unroll
+    for (int b = 0; b < RB; ++b) {
+        if (!live[b]) continue;
+        float h[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) h[i] = grouped_silu(ag[b][i]) * au[b][i];
+        store4(hid + (size_t)slot[b] * ff + n0, h, ff - n0, ff % 4 == 0);
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// down product: float32 rows in the order of the slots
+// ---------------------------------------------------------------------------------------------
+template <int RB>
+__global__ void __launch_bounds__(256) moe_down_grouped_kernel(const bf16_t* __restrict__ hid, const int* __restrict__ order,
+                                                                const int* __restrict__ tile_expert,
+                                                                const int* __restrict__ num_tiles,
+                                                                const bf16_t* __restrict__ down_t, float* __restrict__ part,
+                                                                int D, int ff) {
+    const int tile = blockIdx.y;
+    if (tile >= *num_tiles) return;
+    const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
+    const int r = lane % 16, c = lane / 16;
+    const int nb = blockIdx.x * 4 + wave;             // the wave's block of 16 output columns
+    const int nblocks = (D + 15) / 16, kblocks = (ff + 127) / 128;
+    if (nb >= nblocks) return;
+    const int e = tile_expert[tile];
+    const bf16_t* wd = down_t + ((size_t)e * nblocks + nb) * kblocks * 2048 + lane * 8;
+    const bf16_t* hr[RB];
+    int slot[RB];
+    bool live[RB];
+#pragma unroll
+    for (int b = 0; b < RB; ++b) {
+        slot[b] = (tile * RB + b) * 16 + r;
+        live[b] = order[slot[b]] >= 0;
+        hr[b] = hid + (size_t)(live[b] ? slot[b] : tile * RB * 16) * ff + c * 32;    // (the tile's first slot always has a pair)
+    }
+    f32x4 acc[RB];
+#pragma unroll
+    for (int b = 0; b < RB; ++b) acc[b] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    const int whole = ff / 128;
+    for (int kb = 0; kb < whole; ++kb) {
+        Frag fw[4], fh[RB][4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            fw[j] = frag_load(wd + (size_t)kb * 2048 + j * 512);
+#pragma unroll
+            for (int b = 0; b < RB; ++b) fh[b][j] = frag_load(hr[b] + kb * 128 + j * 8);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int b = 0; b < RB; ++b)
+                acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fw[j].v, fh[b][j].v, acc[b], 0, 0, 0);
+    }
+    if (whole < kblocks) {
+        const int kb = whole;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const Frag fw = frag_load(wd + (size_t)kb * 2048 + j * 512);
+            const bool ok = kb * 128 + c * 32 + j * 8 + 8 <= ff;
+#pragma unroll
+            for (int b = 0; b < RB; ++b) {
+                const Frag fh = frag_load_if(hr[b] + kb * 128 + j * 8, ok);
+                acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fw.v, fh.v, acc[b], 0, 0, 0);
+            }
+        }
+    }
+    const int n0 = nb * 16 + c * 4;
+#pragma unroll
+    for (int b = 0; b < RB; ++b) {
+        if (!live[b]) continue;
+        const float v[4] = {acc[b][0], acc[b][1], acc[b][2], acc[b][3]};
+        store4(part + (size_t)slot[b] * D + n0, v, D - n0, D % 4 == 0);
+    }
+}
+
+// y[row] = sum_j weight[row, j] part[pos[row, j]] (+ gate[row] * shared[row])
+__global__ void moe_combine_kernel(const float* __restrict__ part, const int* __restrict__ pos,
+                                   const float* __restrict__ weights, const bf16_t* __restrict__ shared,
+                                   const float* __restrict__ shared_gate, bf16_t* __restrict__ out, int top, int D) {
+    const int t = blockIdx.x;
+    for (int cidx = threadIdx.x; cidx < D; cidx += blockDim.x) {
+        float y = 0.f;
+        for (int j = 0; j < top; ++j)
+            y = fmaf(weights[(size_t)t * top + j], part[(size_t)pos[(size_t)t * top + j] * D + cidx], y);
+        if (shared) y = fmaf(shared_gate[t], bf16_to_f32(shared[(size_t)t * D + cidx]), y);
+        out[(size_t)t * D + cidx] = f32_to_bf16(y);
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// C ABI
+// ---------------------------------------------------------------------------------------------
+// How many slots a tile has for `pairs` pairs over `experts` experts: 16, 32 or 64 (more rows a tile
+// read an expert's matrices fewer times; fewer waste less on experts with few pairs).
+extern "C" int tli_moe_grouped_tile(int pairs, int experts) {
+    const int average = pairs / (experts > 0 ? experts : 1);
+    return average >= 48 ? 64 : average >= 24 ? 32 : 16;
+}
+
+// scratch, all given by the caller: order [tiles_max * RT], pos [pairs], tile_expert [tiles_max],
+// num_tiles [1] (int32); hid [tiles_max * RT, ff] (bfloat16); part [tiles_max * RT, D] (float32);
+// with tiles_max = pairs / RT + experts.  gate_t, up_t: [E] tiled [ff, D]; down_t: [E] tiled [D, ff].
+extern "C" int tli_moe_grouped_bf16(const void* x, const int* ids, const float* weights, const void* gate_t,
+                                    const void* up_t, const void* down_t, int* order, int* pos, int* tile_expert,
+                                    int* num_tiles, void* hid, float* part, const void* shared,
+                                    const float* shared_gate, void* out, int T, int top, int E, int D, int ff, int RT,
+                                    void* stream) {
+    if (T <= 0) return 0;
+    if (top <= 0 || E <= 0 || E > SORT_MAX_EXPERTS || D <= 0 || ff <= 0 || D % 8 || ff % 8)
+        return tli_fail("moe_grouped: bad sizes (experts %d (at most %d), width %d and hidden units %d in eights)", E,
+                        SORT_MAX_EXPERTS, D, ff);
+    if (RT != 16 && RT != 32 && RT != 64) return tli_fail("moe_grouped: tiles of 16, 32 or 64 slots, not %d", RT);
+    if (shared && !shared_gate) return tli_fail("moe_grouped: a shared expert without its gate");
+    const long long pairs = (long long)T * top;
+    const long long tiles_max = pairs / RT + E;
+    if (tiles_max > 65535 || pairs > (1 << 28)) return tli_fail("moe_grouped: too many pairs for one launch (%lld)", pairs);
+    hipStream_t s = (hipStream_t)stream;
+    hipLaunchKernelGGL(moe_sort_kernel, dim3(1), dim3(1024), 0, s, ids, (int)pairs, E, RT, (int)tiles_max, order, pos,
+                       tile_expert, num_tiles);
+    const dim3 g1((ff + 63) / 64, (unsigned)tiles_max), g2((D + 63) / 64, (unsigned)tiles_max);
+#define TLI_GROUPED(RB)                                                                                              \
+    hipLaunchKernelGGL((moe_gate_up_kernel<RB>), g1, dim3(256), 0, s, (const bf16_t*)x, order, tile_expert, num_tiles, \
+                       (const bf16_t*)gate_t, (const bf16_t*)up_t, (bf16_t*)hid, top, D, ff);                        \
+    hipLaunchKernelGGL((moe_down_grouped_kernel<RB>), g2, dim3(256), 0, s, (const bf16_t*)hid, order, tile_expert,    \
+                       num_tiles, (const bf16_t*)down_t, part, D, ff)
+    if (RT == 16) { TLI_GROUPED(1); }
+    else if (RT == 32) { TLI_GROUPED(2); }
+    else { TLI_GROUPED(4); }
+#undef TLI_GROUPED
+    hipLaunchKernelGGL(moe_combine_kernel, dim3(T), dim3(256), 0, s, part, pos, weights, (const bf16_t*)shared, shared_gate,
+                       (bf16_t*)out, top, D);
+    return tli_check_launch("moe_grouped");
+}

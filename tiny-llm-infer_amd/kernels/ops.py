@@ -109,6 +109,8 @@ def load_library():
         "tli_gated_rmsnorm": [P, P, I, P, P, I, I, I, F, I, P],
         "tli_moe_route": [P, I, P, P, P, I, I, I, I, I, F, I, P],
         "tli_moe_experts": [P, P, P, P, P, P, P, P, P, I, I, I, I, I, P],
+        "tli_moe_grouped_tile": [I, I],
+        "tli_moe_grouped_bf16": [P, P, P, P, P, P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, P],
         "tli_sample": [P, I, I, P, P, P, P, P, P],
         "tli_sample_scratch_bytes": [I],
         "tli_random_normal": [P, ctypes.c_longlong, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint32, P, F, F, I, P],
@@ -199,6 +201,7 @@ class HipOps:
         self.measured = {}           # (rows rounded up to 128, N, K, gated) -> True where gemm_rows won
         self._cold = None            # what is written between two timed runs
         self.attention_tile_rows = 16   # measurements, tests: 32 = tiles of 32 rows in the biased attention kernel (heads up to 128)
+        self.moe_tile = 0            # measurements, tests: force the slots of a tile of the routed experts' products (16, 32, 64)
         self.rows_cfg = 0            # measurements: force a launch shape and the k ranges of gemm_rows
         self.rows_splits = 0
 
@@ -1141,8 +1144,17 @@ class HipOps:
             raise KernelError("a row, or the hidden units of a row's experts, do not fit a workgroup's memory")
 
     def pack_experts(self, w_gate_up, w_down):
-        """Whatever other layout of the experts' matrices the kernels for many rows want (none yet)."""
-        return None
+        """The experts' matrices in the tiled layout that the matrix-core kernels read (``tile_matrix`` of every
+        expert's gate, up and down matrix), or None where those kernels do not apply (float32, sizes that are no
+        multiples of 8, the plain kernels asked for): then ``apply_experts`` works from the row-major matrices."""
+        E, two_ff, n = w_gate_up.shape
+        ff = two_ff // 2
+        if w_gate_up.dtype != torch.bfloat16 or n % 8 or ff % 8 or E > 2048 or self.plain_products:
+            return None
+        return {"gate": torch.stack([self.tile_matrix(w_gate_up[e, :ff]) for e in range(E)]),
+                "up": torch.stack([self.tile_matrix(w_gate_up[e, ff:]) for e in range(E)]),
+                "down": torch.stack([self.tile_matrix(w_down[e]) for e in range(E)]),
+                "experts": E, "hidden": n, "inter": ff}
 
     def route_experts(self, z, experts, top, groups, keep, scale, has_shared):
         """From router logits ``z`` (float32 [T, E (+ 1)]) to the chosen experts (int32 [T, top]), their
@@ -1158,19 +1170,51 @@ class HipOps:
 
     def apply_experts(self, x, ids, weights, w_gate_up, w_down, packed, shared, shared_gate):
         """sum_j weights[t, j] * expert ids[t, j] (x[t])  (+ shared_gate[t] * shared[t]);  ``w_gate_up``
-        [E, 2 ff, n] (an expert's gate rows, then its up rows), ``w_down`` [E, n, ff]."""
+        [E, 2 ff, n] (an expert's gate rows, then its up rows), ``w_down`` [E, n, ff]; with ``packed`` (what
+        ``pack_experts`` gave) the row-major matrices may be None."""
         T, n = x.shape
-        E, two_ff, _ = w_gate_up.shape
-        ff, top = two_ff // 2, ids.shape[1]
+        top = ids.shape[1]
         self._want(x, "expert input")
-        self._want(w_gate_up, "experts' gate and up matrices", x.dtype, (E, 2 * ff, n))
-        self._want(w_down, "experts' down matrices", x.dtype, (E, n, ff))
         self._want(ids, "chosen experts", torch.int32, (T, top))
         self._want(weights, "experts' weights", torch.float32, (T, top))
         if shared is not None:
             self._want(shared, "shared expert's output", x.dtype, (T, n))
             self._want(shared_gate, "shared expert's gate", torch.float32, (T,))
         out = torch.empty((T, n), dtype=x.dtype, device=self.device)
+        if T == 0:
+            return out
+        if packed is not None and x.dtype == torch.bfloat16 and not self.plain_products:
+            E, ff = packed["experts"], packed["inter"]
+            if packed["hidden"] != n:
+                raise KernelError(f"the experts read rows of {packed['hidden']}, the input has {n}")
+            nb, kb = (ff + 15) // 16, (n + 127) // 128
+            for role, shape in (("gate", (E, nb, kb, 4, 4, 16, 8)), ("up", (E, nb, kb, 4, 4, 16, 8)),
+                                ("down", (E, (n + 15) // 16, (ff + 127) // 128, 4, 4, 16, 8))):
+                self._want(packed[role], f"experts' {role} matrices (tiled)", torch.bfloat16, shape)
+            a_call = max(1, (65535 - E) * 16 // top)                 # (a launch's grid holds 65,535 tiles)
+            for t0 in range(0, T, a_call):
+                t1 = min(T, t0 + a_call)
+                pairs = (t1 - t0) * top
+                RT = self.moe_tile or int(self.lib.tli_moe_grouped_tile(pairs, E))
+                slots = (pairs // RT + E) * RT
+                i32 = dict(dtype=torch.int32, device=self.device)
+                order, pos = torch.empty((slots,), **i32), torch.empty((pairs,), **i32)
+                tile_expert, num_tiles = torch.empty((slots // RT,), **i32), torch.empty((1,), **i32)
+                hid = torch.empty((slots, ff), dtype=torch.bfloat16, device=self.device)
+                part = torch.empty((slots, n), dtype=torch.float32, device=self.device)
+                self._call(self.lib.tli_moe_grouped_bf16, x[t0:t1].data_ptr(), ids[t0:t1].data_ptr(), weights[t0:t1].data_ptr(),
+                           packed["gate"].data_ptr(), packed["up"].data_ptr(), packed["down"].data_ptr(), order.data_ptr(),
+                           pos.data_ptr(), tile_expert.data_ptr(), num_tiles.data_ptr(), hid.data_ptr(), part.data_ptr(),
+                           None if shared is None else shared[t0:t1].data_ptr(),
+                           None if shared is None else shared_gate[t0:t1].data_ptr(), out[t0:t1].data_ptr(), t1 - t0, top,
+                           E, n, ff, RT, self._stream())
+            return out
+        if w_gate_up is None or w_down is None:
+            raise KernelError("the experts' row-major matrices were not kept and the tiled ones do not apply here")
+        E, two_ff, _ = w_gate_up.shape
+        ff = two_ff // 2
+        self._want(w_gate_up, "experts' gate and up matrices", x.dtype, (E, 2 * ff, n))
+        self._want(w_down, "experts' down matrices", x.dtype, (E, n, ff))
         hid = torch.empty((T * top, ff), dtype=x.dtype, device=self.device)
         for t0 in range(0, T, 32768):
             t1 = min(T, t0 + 32768)

@@ -69,7 +69,11 @@ class RoutedExperts(FeedForward):
         self.w_gate_up = torch.stack([torch.cat([weights[self._expert(j, "gate")], weights[self._expert(j, "up")]], dim=0)
                                       for j in range(self.experts)]).to(env.dtype).contiguous()
         self.w_down = torch.stack([weights[self._expert(j, "down")] for j in range(self.experts)]).to(env.dtype).contiguous()
+        # (where the kernels for the matrix cores apply they read a layout of their own, and the row-major
+        # matrices are not kept beside it)
         self.packed = env.ops.pack_experts(self.w_gate_up, self.w_down)
+        if self.packed is not None:
+            self.w_gate_up = self.w_down = None
         self.shared_gate_up = self.shared_down = None
         if self.shared_inter is not None:
             self.shared_gate_up = GatedMatrix(weights[n["shared_gate"]], weights[n["shared_up"]], env)
