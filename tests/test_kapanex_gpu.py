@@ -169,7 +169,7 @@ def test_router_choice_and_weights(ops, E, top, groups, keep):
     assert none is None and torch.equal(ids2, ids) and torch.equal(wts2, wts)
 
 
-@pytest.mark.parametrize("dtype", ["float32", "bfloat16", "bfloat16-plain", "bfloat16-tiles-of-16", "bfloat16-tiles-of-64"])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16", "bfloat16-plain", "bfloat16-tiles-of-16", "bfloat16-tiles-of-64", "bfloat16-tiles-of-128"])
 @pytest.mark.parametrize("T, E, top, n, ff", [(1, 4, 1, 48, 40), (5, 6, 2, 64, 32), (40, 8, 3, 100, 24), (300, 16, 4, 128, 64),
                                               (700, 8, 2, 256, 96), (130, 3, 3, 136, 200)])
 def test_chosen_experts_applied_and_added(ops, dtype, T, E, top, n, ff):

@@ -122,9 +122,19 @@ __global__ __launch_bounds__(256) void delta_recurrence_kernel(
     const float* __restrict__ beta, const float* __restrict__ decay, const float* __restrict__ qk,
     float* __restrict__ state, float* __restrict__ out, const int* __restrict__ row_start,
     const int* __restrict__ seq_start, const int* __restrict__ slots, int H, int G, int dk, int dv) {
+    // A sequence's rows pass through LDS in chunks of CT: the whole workgroup fetches a chunk with loads that
+    // do not wait for each other (into registers, while the chunk before is worked on), so the walk along the
+    // rows waits for LDS only.  In LDS an element i = part + 8 r of k or q lies at part * RPT + r: a lane's
+    // share of a row is one run.
+    constexpr int CT = RPT == 32 ? 16 : 32;      // rows a chunk (k and q of a chunk: 2 * CT * 8 RPT floats)
+    constexpr int DKP = DELTA_LANES * RPT;
+    constexpr int NK = CT * RPT / 32;            // elements of k (and of q) a thread fetches a chunk
+    constexpr int NV = CT / 8;                   // of v
+    __shared__ float ks[CT * DKP], qs[CT * DKP], vs[CT * DELTA_COLS], sc[3 * CT];
     const int seq = blockIdx.z, head = blockIdx.y;
     const int part = threadIdx.x % DELTA_LANES;
-    const int col_raw = blockIdx.x * DELTA_COLS + threadIdx.x / DELTA_LANES;
+    const int local = threadIdx.x / DELTA_LANES;
+    const int col_raw = blockIdx.x * DELTA_COLS + local;
     const bool live = col_raw < dv;
     const int col = live ? col_raw : dv - 1;
     const int kvh = head / (H / G);
@@ -138,44 +148,65 @@ __global__ __launch_bounds__(256) void delta_recurrence_kernel(
         S[r] = (!fresh && i < dk) ? mine[(size_t)i * dv + col] : 0.f;
     }
     const size_t qd = (size_t)G * dk, vd = (size_t)H * dv;
-    float k[RPT], q[RPT], kx[RPT], qx[RPT];
-    float v = 0.f, b = 0.f, g = 0.f, c = 0.f;
-    // the row after the current one is asked for while the current one is worked on
-    auto load = [&](int t, float (&kk)[RPT], float (&qq)[RPT], float& vv, float& bb, float& gg, float& cc) {
-        const float* kp = kn + (size_t)t * qd + (size_t)kvh * dk;
-        const float* qp = qn + (size_t)t * qd + (size_t)kvh * dk;
+    float pk[NK], pq[NK], pv[NV], ps = 0.f;
+    auto fetch = [&](int c0) {                   // the chunk that starts at row c0, into registers
 #pragma unroll
-        for (int r = 0; r < RPT; ++r) {
-            const int i = part + DELTA_LANES * r;
-            kk[r] = i < dk ? kp[i] : 0.f;
-            qq[r] = i < dk ? qp[i] : 0.f;
+        for (int n = 0; n < NK; ++n) {
+            const int e = threadIdx.x + n * 256, t = e / DKP, i = e % DKP;
+            const bool ok = c0 + t < r1 && i < dk;
+            pk[n] = ok ? kn[(size_t)(c0 + t) * qd + (size_t)kvh * dk + i] : 0.f;
+            pq[n] = ok ? qn[(size_t)(c0 + t) * qd + (size_t)kvh * dk + i] : 0.f;
         }
-        vv = vc[(size_t)t * vd + (size_t)head * dv + col];
-        bb = beta[(size_t)t * H + head];
-        gg = decay[(size_t)t * H + head];
-        cc = qk[(size_t)t * G + kvh];
+#pragma unroll
+        for (int n = 0; n < NV; ++n) {
+            const int e = threadIdx.x + n * 256, t = e / DELTA_COLS, j = blockIdx.x * DELTA_COLS + e % DELTA_COLS;
+            pv[n] = (c0 + t < r1 && j < dv) ? vc[(size_t)(c0 + t) * vd + (size_t)head * dv + j] : 0.f;
+        }
+        if (threadIdx.x < 3 * CT) {
+            const int which = threadIdx.x / CT, t = threadIdx.x % CT;
+            if (c0 + t < r1)
+                ps = which == 0 ? beta[(size_t)(c0 + t) * H + head]
+                                : which == 1 ? decay[(size_t)(c0 + t) * H + head] : qk[(size_t)(c0 + t) * G + kvh];
+        }
     };
-    if (r0 < r1) load(r0, kx, qx, v, b, g, c);
-    for (int t = r0; t < r1; ++t) {
-        const float v0 = v, b0 = b, g0 = g, c0 = c;
+    if (r0 < r1) fetch(r0);
+    for (int c0 = r0; c0 < r1; c0 += CT) {
+        __syncthreads();                         // the chunk before has been walked
 #pragma unroll
-        for (int r = 0; r < RPT; ++r) { k[r] = kx[r]; q[r] = qx[r]; }
-        if (t + 1 < r1) load(t + 1, kx, qx, v, b, g, c);
-        float d1 = 0.f, d2 = 0.f;
-#pragma unroll
-        for (int r = 0; r < RPT; ++r) {
-            d1 = fmaf(k[r], S[r], d1);
-            d2 = fmaf(q[r], S[r], d2);
+        for (int n = 0; n < NK; ++n) {
+            const int e = threadIdx.x + n * 256, t = e / DKP, i = e % DKP;
+            const int at = t * DKP + (i % DELTA_LANES) * RPT + i / DELTA_LANES;
+            ks[at] = pk[n];
+            qs[at] = pq[n];
         }
 #pragma unroll
-        for (int off = 1; off < DELTA_LANES; off <<= 1) {
-            d1 += __shfl_xor(d1, off, TLI_WAVE);
-            d2 += __shfl_xor(d2, off, TLI_WAVE);
-        }
-        const float u = b0 * (v0 - g0 * d1);
+        for (int n = 0; n < NV; ++n) vs[threadIdx.x + n * 256] = pv[n];
+        if (threadIdx.x < 3 * CT) sc[threadIdx.x] = ps;
+        __syncthreads();
+        if (c0 + CT < r1) fetch(c0 + CT);
+        const int rows = min(CT, r1 - c0);
+        for (int t = 0; t < rows; ++t) {
+            const float* kp = ks + t * DKP + part * RPT;
+            const float* qp = qs + t * DKP + part * RPT;
+            float k[RPT];
+            float d1 = 0.f, d2 = 0.f;
 #pragma unroll
-        for (int r = 0; r < RPT; ++r) S[r] = fmaf(k[r], u, g0 * S[r]);
-        if (part == 0 && live) out[(size_t)t * vd + (size_t)head * dv + col] = fmaf(c0, u, g0 * d2);
+            for (int r = 0; r < RPT; ++r) {
+                k[r] = kp[r];
+                d1 = fmaf(k[r], S[r], d1);
+                d2 = fmaf(qp[r], S[r], d2);
+            }
+#pragma unroll
+            for (int off = 1; off < DELTA_LANES; off <<= 1) {
+                d1 += __shfl_xor(d1, off, TLI_WAVE);
+                d2 += __shfl_xor(d2, off, TLI_WAVE);
+            }
+            const float g0 = sc[CT + t];
+            const float u = sc[t] * (vs[t * DELTA_COLS + local] - g0 * d1);
+#pragma unroll
+            for (int r = 0; r < RPT; ++r) S[r] = fmaf(k[r], u, g0 * S[r]);
+            if (part == 0 && live) out[(size_t)(c0 + t) * vd + (size_t)head * dv + col] = fmaf(sc[2 * CT + t], u, g0 * d2);
+        }
     }
     if (live) {
 #pragma unroll

@@ -15,7 +15,7 @@
 // KiB, in the order the operands of v_mfma_f32_16x16x32_bf16 want: a load instruction of a wave takes 1 KiB
 // in a row); rows and columns that do not exist are zeros there.  A is a tile of W (16 outputs), B the
 // rows of x, so a lane ends with 4 consecutive outputs of one row.  A wave takes 16 outputs and all RT
-// rows of its tile; the four waves of a workgroup share the rows of x through the cache.
+// rows of its tile; the four waves of a workgroup share the rows of x through LDS.
 #include "common.h"
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
@@ -30,11 +30,6 @@ union Frag {
 __device__ __forceinline__ Frag frag_load(const bf16_t* p) {
     Frag f;
     f.u = *reinterpret_cast<const uint4*>(p);
-    return f;
-}
-__device__ __forceinline__ Frag frag_load_if(const bf16_t* p, bool ok) {
-    Frag f;
-    f.u = ok ? *reinterpret_cast<const uint4*>(p) : make_uint4(0, 0, 0, 0);
     return f;
 }
 
@@ -79,150 +74,125 @@ __global__ void __launch_bounds__(1024) moe_sort_kernel(const int* __restrict__ 
 }
 
 // ---------------------------------------------------------------------------------------------
-// gate and up products with the activation
+// one tile's product: 16 RB rows of B against the wave's 16 rows of A (and of A2, if GATED)
 // ---------------------------------------------------------------------------------------------
+#define XT_STRIDE 136          // bfloat16 elements between two rows of the staged block of B: 128 and 8 more, so that
+                               // the 16 rows a quarter of a wave reads lie in different banks
+
+// The four waves of a workgroup read the same rows of B: a block of 128 columns of them is staged in
+// LDS by all threads together (rows without a pair, and columns past the end, as zeros), then every
+// wave takes its fragments from there.  `src_off`: for each of the tile's rows the offset of its
+// source row, or a negative number.
+template <int RB, bool GATED>
+__device__ __forceinline__ void tile_product(const bf16_t* __restrict__ a1, const bf16_t* __restrict__ a2,
+                                             const bf16_t* __restrict__ src, const long long* src_off, int K, bool active,
+                                             bf16_t* xt, f32x4 (&acc1)[RB], f32x4 (&acc2)[RB]) {
+    const int lane = threadIdx.x % 64, r = lane % 16, c = lane / 16;
+    const int kblocks = (K + 127) / 128;
+    for (int kb = 0; kb < kblocks; ++kb) {
+        __syncthreads();
+#pragma unroll
+        for (int n = 0; n < RB; ++n) {
+            const int id = threadIdx.x + n * 256, row = id / 16, kc = id % 16;
+            const long long off = src_off[row];
+            const int k = kb * 128 + kc * 8;
+            uint4 v = make_uint4(0, 0, 0, 0);
+            if (off >= 0 && k + 8 <= K) v = *reinterpret_cast<const uint4*>(src + off + k);
+            *reinterpret_cast<uint4*>(xt + row * XT_STRIDE + kc * 8) = v;
+        }
+        __syncthreads();
+        if (!active) continue;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const Frag f1 = frag_load(a1 + (size_t)kb * 2048 + j * 512);
+            Frag f2;
+            if (GATED) f2 = frag_load(a2 + (size_t)kb * 2048 + j * 512);
+#pragma unroll
+            for (int b = 0; b < RB; ++b) {
+                Frag fx;
+                fx.u = *reinterpret_cast<const uint4*>(xt + (b * 16 + r) * XT_STRIDE + c * 32 + j * 8);
+                acc1[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f1.v, fx.v, acc1[b], 0, 0, 0);
+                if (GATED) acc2[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f2.v, fx.v, acc2[b], 0, 0, 0);
+            }
+        }
+    }
+}
+
 __device__ __forceinline__ float grouped_silu(float z) { return z / (1.0f + expf(-z)); }
 
-template <int RB>            // a tile has 16 RB slots
+// gate and up products with the activation: hid[slot, f] (a tile has 16 RB slots)
+template <int RB>
 __global__ void __launch_bounds__(256) moe_gate_up_kernel(const bf16_t* __restrict__ x, const int* __restrict__ order,
                                                            const int* __restrict__ tile_expert,
                                                            const int* __restrict__ num_tiles,
                                                            const bf16_t* __restrict__ gate_t,
                                                            const bf16_t* __restrict__ up_t, bf16_t* __restrict__ hid,
                                                            int top, int D, int ff) {
+    __shared__ __attribute__((aligned(16))) bf16_t xt[16 * RB * XT_STRIDE];
+    __shared__ long long src_off[16 * RB];
     const int tile = blockIdx.y;
-    if (tile >= *num_tiles) return;
+    if (tile >= *num_tiles) return;                   // (the whole workgroup)
     const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
     const int r = lane % 16, c = lane / 16;
     const int nb = blockIdx.x * 4 + wave;             // the wave's block of 16 hidden units
     const int nblocks = (ff + 15) / 16, kblocks = (D + 127) / 128;
-    if (nb >= nblocks) return;
+    const bool active = nb < nblocks;
     const int e = tile_expert[tile];
-    const size_t block0 = ((size_t)e * nblocks + nb) * kblocks * 2048 + lane * 8;
-    const bf16_t* wg = gate_t + block0;
-    const bf16_t* wu = up_t + block0;
-    const bf16_t* xr[RB];
-    int slot[RB];
-    bool live[RB];
-#pragma unroll
-    for (int b = 0; b < RB; ++b) {
-        slot[b] = (tile * RB + b) * 16 + r;
-        const int p = order[slot[b]];
-        live[b] = p >= 0;
-        xr[b] = x + (size_t)(live[b] ? p / top : 0) * D + c * 32;       // (a slot without a pair reads row 0 and stores nothing)
+    for (int i = threadIdx.x; i < 16 * RB; i += 256) {
+        const int p = order[tile * 16 * RB + i];
+        src_off[i] = p >= 0 ? (long long)(p / top) * D : -1;
     }
+    const size_t block0 = ((size_t)e * nblocks + (active ? nb : 0)) * kblocks * 2048 + lane * 8;
     f32x4 ag[RB], au[RB];
 #pragma unroll
     for (int b = 0; b < RB; ++b) ag[b] = au[b] = (f32x4){0.f, 0.f, 0.f, 0.f};
-    const int whole = D / 128;
-    for (int kb = 0; kb < whole; ++kb) {
-        Frag fg[4], fu[4], fx[RB][4];
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            fg[j] = frag_load(wg + (size_t)kb * 2048 + j * 512);
-            fu[j] = frag_load(wu + (size_t)kb * 2048 + j * 512);
-#pragma unroll
-            for (int b = 0; b < RB; ++b) fx[b][j] = frag_load(xr[b] + kb * 128 + j * 8);
-        }
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-#pragma unroll
-            for (int b = 0; b < RB; ++b) {
-                ag[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fg[j].v, fx[b][j].v, ag[b], 0, 0, 0);
-                au[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fu[j].v, fx[b][j].v, au[b], 0, 0, 0);
-            }
-    }
-    if (whole < kblocks) {                            // the last, partial block of k: rows of x end before it does
-        const int kb = whole;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const Frag fg = frag_load(wg + (size_t)kb * 2048 + j * 512);
-            const Frag fu = frag_load(wu + (size_t)kb * 2048 + j * 512);
-            const bool ok = kb * 128 + c * 32 + j * 8 + 8 <= D;
-#pragma unroll
-            for (int b = 0; b < RB; ++b) {
-                const Frag fx = frag_load_if(xr[b] + kb * 128 + j * 8, ok);
-                ag[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fg.v, fx.v, ag[b], 0, 0, 0);
-                au[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fu.v, fx.v, au[b], 0, 0, 0);
-            }
-        }
-    }
+    tile_product<RB, true>(gate_t + block0, up_t + block0, x, src_off, D, active, xt, ag, au);
+    if (!active) return;
     // the lane holds hidden units nb * 16 + 4 c .. + 4 of the slots 16 b + r
     const int n0 = nb * 16 + c * 4;
 #pragma unroll
     for (int b = 0; b < RB; ++b) {
-        if (!live[b]) continue;
+        if (src_off[b * 16 + r] < 0) continue;
         float h[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) h[i] = grouped_silu(ag[b][i]) * au[b][i];
-        store4(hid + (size_t)slot[b] * ff + n0, h, ff - n0, ff % 4 == 0);
+        store4(hid + (size_t)((tile * RB + b) * 16 + r) * ff + n0, h, ff - n0, ff % 4 == 0);
     }
 }
 
-// ---------------------------------------------------------------------------------------------
 // down product: float32 rows in the order of the slots
-// ---------------------------------------------------------------------------------------------
 template <int RB>
 __global__ void __launch_bounds__(256) moe_down_grouped_kernel(const bf16_t* __restrict__ hid, const int* __restrict__ order,
                                                                 const int* __restrict__ tile_expert,
                                                                 const int* __restrict__ num_tiles,
                                                                 const bf16_t* __restrict__ down_t, float* __restrict__ part,
                                                                 int D, int ff) {
+    __shared__ __attribute__((aligned(16))) bf16_t xt[16 * RB * XT_STRIDE];
+    __shared__ long long src_off[16 * RB];
     const int tile = blockIdx.y;
     if (tile >= *num_tiles) return;
     const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
     const int r = lane % 16, c = lane / 16;
     const int nb = blockIdx.x * 4 + wave;             // the wave's block of 16 output columns
     const int nblocks = (D + 15) / 16, kblocks = (ff + 127) / 128;
-    if (nb >= nblocks) return;
+    const bool active = nb < nblocks;
     const int e = tile_expert[tile];
-    const bf16_t* wd = down_t + ((size_t)e * nblocks + nb) * kblocks * 2048 + lane * 8;
-    const bf16_t* hr[RB];
-    int slot[RB];
-    bool live[RB];
-#pragma unroll
-    for (int b = 0; b < RB; ++b) {
-        slot[b] = (tile * RB + b) * 16 + r;
-        live[b] = order[slot[b]] >= 0;
-        hr[b] = hid + (size_t)(live[b] ? slot[b] : tile * RB * 16) * ff + c * 32;    // (the tile's first slot always has a pair)
+    for (int i = threadIdx.x; i < 16 * RB; i += 256) {
+        const int slot = tile * 16 * RB + i;
+        src_off[i] = order[slot] >= 0 ? (long long)slot * ff : -1;
     }
-    f32x4 acc[RB];
+    const bf16_t* wd = down_t + ((size_t)e * nblocks + (active ? nb : 0)) * kblocks * 2048 + lane * 8;
+    f32x4 acc[RB], unused[RB];
 #pragma unroll
     for (int b = 0; b < RB; ++b) acc[b] = (f32x4){0.f, 0.f, 0.f, 0.f};
-    const int whole = ff / 128;
-    for (int kb = 0; kb < whole; ++kb) {
-        Frag fw[4], fh[RB][4];
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            fw[j] = frag_load(wd + (size_t)kb * 2048 + j * 512);
-#pragma unroll
-            for (int b = 0; b < RB; ++b) fh[b][j] = frag_load(hr[b] + kb * 128 + j * 8);
-        }
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-#pragma unroll
-            for (int b = 0; b < RB; ++b)
-                acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fw[j].v, fh[b][j].v, acc[b], 0, 0, 0);
-    }
-    if (whole < kblocks) {
-        const int kb = whole;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const Frag fw = frag_load(wd + (size_t)kb * 2048 + j * 512);
-            const bool ok = kb * 128 + c * 32 + j * 8 + 8 <= ff;
-#pragma unroll
-            for (int b = 0; b < RB; ++b) {
-                const Frag fh = frag_load_if(hr[b] + kb * 128 + j * 8, ok);
-                acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fw.v, fh.v, acc[b], 0, 0, 0);
-            }
-        }
-    }
+    tile_product<RB, false>(wd, nullptr, hid, src_off, ff, active, xt, acc, unused);
+    if (!active) return;
     const int n0 = nb * 16 + c * 4;
 #pragma unroll
     for (int b = 0; b < RB; ++b) {
-        if (!live[b]) continue;
+        if (src_off[b * 16 + r] < 0) continue;
         const float v[4] = {acc[b][0], acc[b][1], acc[b][2], acc[b][3]};
-        store4(part + (size_t)slot[b] * D + n0, v, D - n0, D % 4 == 0);
+        store4(part + (size_t)((tile * RB + b) * 16 + r) * D + n0, v, D - n0, D % 4 == 0);
     }
 }
 
@@ -243,11 +213,11 @@ __global__ void moe_combine_kernel(const float* __restrict__ part, const int* __
 // ---------------------------------------------------------------------------------------------
 // C ABI
 // ---------------------------------------------------------------------------------------------
-// How many slots a tile has for `pairs` pairs over `experts` experts: 16, 32 or 64 (more rows a tile
+// How many slots a tile has for `pairs` pairs over `experts` experts: 16, 32, 64 or 128 (more rows a tile
 // read an expert's matrices fewer times; fewer waste less on experts with few pairs).
 extern "C" int tli_moe_grouped_tile(int pairs, int experts) {
     const int average = pairs / (experts > 0 ? experts : 1);
-    return average >= 48 ? 64 : average >= 24 ? 32 : 16;
+    return average >= 96 ? 128 : average >= 48 ? 64 : average >= 24 ? 32 : 16;
 }
 
 // scratch, all given by the caller: order [tiles_max * RT], pos [pairs], tile_expert [tiles_max],
@@ -262,7 +232,8 @@ extern "C" int tli_moe_grouped_bf16(const void* x, const int* ids, const float* 
     if (top <= 0 || E <= 0 || E > SORT_MAX_EXPERTS || D <= 0 || ff <= 0 || D % 8 || ff % 8)
         return tli_fail("moe_grouped: bad sizes (experts %d (at most %d), width %d and hidden units %d in eights)", E,
                         SORT_MAX_EXPERTS, D, ff);
-    if (RT != 16 && RT != 32 && RT != 64) return tli_fail("moe_grouped: tiles of 16, 32 or 64 slots, not %d", RT);
+    if (RT != 16 && RT != 32 && RT != 64 && RT != 128)
+        return tli_fail("moe_grouped: tiles of 16, 32, 64 or 128 slots, not %d", RT);
     if (shared && !shared_gate) return tli_fail("moe_grouped: a shared expert without its gate");
     const long long pairs = (long long)T * top;
     const long long tiles_max = pairs / RT + E;
@@ -278,7 +249,8 @@ extern "C" int tli_moe_grouped_bf16(const void* x, const int* ids, const float* 
                        num_tiles, (const bf16_t*)down_t, part, D, ff)
     if (RT == 16) { TLI_GROUPED(1); }
     else if (RT == 32) { TLI_GROUPED(2); }
-    else { TLI_GROUPED(4); }
+    else if (RT == 64) { TLI_GROUPED(4); }
+    else { TLI_GROUPED(8); }
 #undef TLI_GROUPED
     hipLaunchKernelGGL(moe_combine_kernel, dim3(T), dim3(256), 0, s, part, pos, weights, (const bf16_t*)shared, shared_gate,
                        (bf16_t*)out, top, D);

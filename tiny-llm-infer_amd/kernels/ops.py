@@ -201,7 +201,7 @@ class HipOps:
         self.measured = {}           # (rows rounded up to 128, N, K, gated) -> True where gemm_rows won
         self._cold = None            # what is written between two timed runs
         self.attention_tile_rows = 16   # measurements, tests: 32 = tiles of 32 rows in the biased attention kernel (heads up to 128)
-        self.moe_tile = 0            # measurements, tests: force the slots of a tile of the routed experts' products (16, 32, 64)
+        self.moe_tile = 0            # measurements, tests: force the slots of a tile of the routed experts' products (16, 32, 64, 128)
         self.rows_cfg = 0            # measurements: force a launch shape and the k ranges of gemm_rows
         self.rows_splits = 0
 
