@@ -14,7 +14,7 @@
 // not read.  Everything after the projections is float32.
 //
 // The recurrence walks a sequence's rows one after the other.  Columns of S are independent, so a
-// column belongs to 8 neighbouring lanes, each holding every 8th of its dk elements in registers; the
+// column belongs to 16 neighbouring lanes, each holding every 16th of its dk elements in registers; the
 // two dot products of a row (k'.S and q'.S, both with the old S, since
 // o = decay (q'.S_old) + (q'.k') u) are reduced over those lanes together.
 #include "common.h"
@@ -113,10 +113,20 @@ __global__ void delta_conv_keep_kernel(const T* __restrict__ proj, int ld, T* __
 // ---------------------------------------------------------------------------------------------
 // recurrence
 // ---------------------------------------------------------------------------------------------
-#define DELTA_LANES 8          // lanes that share a column of S
-#define DELTA_COLS 32          // columns a workgroup of 256 threads walks
+#define DELTA_LANES 16         // lanes that share a column of S: one row of 16 lanes, summed over with DPP moves
+#define DELTA_COLS 16          // columns a workgroup of 256 threads walks
 
-template <int RPT>             // elements of a column a lane holds: dk <= 8 * RPT
+// Sum over the 16 lanes of a row, every lane gets it: neighbours, pairs (quad permutations), then the mirror
+// image inside each half row and inside the row (by then the lanes of a quad, of a half row, hold the same).
+__device__ __forceinline__ float row16_sum(float v) {
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xF, 0xF, true));    // quad_perm [1,0,3,2]
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xF, 0xF, true));    // quad_perm [2,3,0,1]
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xF, 0xF, true));   // row_half_mirror
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xF, 0xF, true));   // row_mirror
+    return v;
+}
+
+template <int RPT>             // elements of a column a lane holds: dk <= 16 * RPT
 __global__ __launch_bounds__(256) void delta_recurrence_kernel(
     const float* __restrict__ qn, const float* __restrict__ kn, const float* __restrict__ vc,
     const float* __restrict__ beta, const float* __restrict__ decay, const float* __restrict__ qk,
@@ -124,12 +134,12 @@ __global__ __launch_bounds__(256) void delta_recurrence_kernel(
     const int* __restrict__ seq_start, const int* __restrict__ slots, int H, int G, int dk, int dv) {
     // A sequence's rows pass through LDS in chunks of CT: the whole workgroup fetches a chunk with loads that
     // do not wait for each other (into registers, while the chunk before is worked on), so the walk along the
-    // rows waits for LDS only.  In LDS an element i = part + 8 r of k or q lies at part * RPT + r: a lane's
+    // rows waits for LDS only.  In LDS an element i = part + 16 r of k or q lies at part * RPT + r: a lane's
     // share of a row is one run.
-    constexpr int CT = RPT == 32 ? 16 : 32;      // rows a chunk (k and q of a chunk: 2 * CT * 8 RPT floats)
+    constexpr int CT = RPT == 16 ? 16 : 32;      // rows a chunk (k and q of a chunk: 2 * CT * 16 RPT floats)
     constexpr int DKP = DELTA_LANES * RPT;
-    constexpr int NK = CT * RPT / 32;            // elements of k (and of q) a thread fetches a chunk
-    constexpr int NV = CT / 8;                   // of v
+    constexpr int NK = CT * DKP / 256;           // elements of k (and of q) a thread fetches a chunk
+    constexpr int NV = CT * DELTA_COLS / 256;    // of v
     __shared__ float ks[CT * DKP], qs[CT * DKP], vs[CT * DELTA_COLS], sc[3 * CT];
     const int seq = blockIdx.z, head = blockIdx.y;
     const int part = threadIdx.x % DELTA_LANES;
@@ -185,27 +195,34 @@ __global__ __launch_bounds__(256) void delta_recurrence_kernel(
         __syncthreads();
         if (c0 + CT < r1) fetch(c0 + CT);
         const int rows = min(CT, r1 - c0);
-        for (int t = 0; t < rows; ++t) {
+        // the row after the current one is read from LDS while the current one is worked on
+        float kx[RPT], qx[RPT], vx, bx, gx, cx;
+        auto read_row = [&](int t) {
             const float* kp = ks + t * DKP + part * RPT;
             const float* qp = qs + t * DKP + part * RPT;
-            float k[RPT];
-            float d1 = 0.f, d2 = 0.f;
+#pragma unroll
+            for (int r = 0; r < RPT; ++r) { kx[r] = kp[r]; qx[r] = qp[r]; }
+            vx = vs[t * DELTA_COLS + local];
+            bx = sc[t]; gx = sc[CT + t]; cx = sc[2 * CT + t];
+        };
+        read_row(0);
+        for (int t = 0; t < rows; ++t) {
+            float k[RPT], q[RPT];
+#pragma unroll
+            for (int r = 0; r < RPT; ++r) { k[r] = kx[r]; q[r] = qx[r]; }
+            const float v0 = vx, b0 = bx, g0 = gx, c0q = cx;
+            read_row(min(t + 1, CT - 1));
+            float d1[2] = {0.f, 0.f}, d2[2] = {0.f, 0.f};          // two sums each: shorter chains of dependent additions
 #pragma unroll
             for (int r = 0; r < RPT; ++r) {
-                k[r] = kp[r];
-                d1 = fmaf(k[r], S[r], d1);
-                d2 = fmaf(qp[r], S[r], d2);
+                d1[r & 1] = fmaf(k[r], S[r], d1[r & 1]);
+                d2[r & 1] = fmaf(q[r], S[r], d2[r & 1]);
             }
-#pragma unroll
-            for (int off = 1; off < DELTA_LANES; off <<= 1) {
-                d1 += __shfl_xor(d1, off, TLI_WAVE);
-                d2 += __shfl_xor(d2, off, TLI_WAVE);
-            }
-            const float g0 = sc[CT + t];
-            const float u = sc[t] * (vs[t * DELTA_COLS + local] - g0 * d1);
+            const float s1 = row16_sum(d1[0] + d1[1]), s2 = row16_sum(d2[0] + d2[1]);
+            const float u = b0 * (v0 - g0 * s1);
 #pragma unroll
             for (int r = 0; r < RPT; ++r) S[r] = fmaf(k[r], u, g0 * S[r]);
-            if (part == 0 && live) out[(size_t)(c0 + t) * vd + (size_t)head * dv + col] = fmaf(sc[2 * CT + t], u, g0 * d2);
+            if (part == 0 && live) out[(size_t)(c0 + t) * vd + (size_t)head * dv + col] = fmaf(c0q, u, g0 * s2);
         }
     }
     if (live) {
@@ -296,11 +313,11 @@ extern "C" int tli_delta_recurrence(const float* qn, const float* kn, const floa
     const dim3 grid((dv + DELTA_COLS - 1) / DELTA_COLS, H, seqs);
 #define TLI_DELTA(RPT) hipLaunchKernelGGL((delta_recurrence_kernel<RPT>), grid, dim3(256), 0, s, qn, kn, vc, beta, \
                                           decay, qk, state, out, row_start, seq_start, slots, H, G, dk, dv)
-    if (dk <= 16) TLI_DELTA(2);
-    else if (dk <= 32) TLI_DELTA(4);
-    else if (dk <= 64) TLI_DELTA(8);
-    else if (dk <= 128) TLI_DELTA(16);
-    else TLI_DELTA(32);
+    if (dk <= 16) TLI_DELTA(1);
+    else if (dk <= 32) TLI_DELTA(2);
+    else if (dk <= 64) TLI_DELTA(4);
+    else if (dk <= 128) TLI_DELTA(8);
+    else TLI_DELTA(16);
 #undef TLI_DELTA
     return tli_check_launch("delta_recurrence");
 }

@@ -14,7 +14,7 @@
 // The matrices are read in the tiled layout of the other products (blocks of 16 rows x 128 columns, 4
 // KiB, in the order the operands of v_mfma_f32_16x16x32_bf16 want: a load instruction of a wave takes 1 KiB
 // in a row); rows and columns that do not exist are zeros there.  A is a tile of W (16 outputs), B the
-// rows of x, so a lane ends with 4 consecutive outputs of one row.  A wave takes 16 outputs and all RT
+// rows of x, so a lane ends with 4 consecutive outputs of one row.  A wave takes 32 outputs and all RT
 // rows of its tile; the four waves of a workgroup share the rows of x through LDS.
 #include "common.h"
 
@@ -83,10 +83,12 @@ __global__ void __launch_bounds__(1024) moe_sort_kernel(const int* __restrict__ 
 // LDS by all threads together (rows without a pair, and columns past the end, as zeros), then every
 // wave takes its fragments from there.  `src_off`: for each of the tile's rows the offset of its
 // source row, or a negative number.
+#define NB 2                   // blocks of 16 outputs a wave takes: a fragment of B from LDS serves that many products
+
 template <int RB, bool GATED>
-__device__ __forceinline__ void tile_product(const bf16_t* __restrict__ a1, const bf16_t* __restrict__ a2,
+__device__ __forceinline__ void tile_product(const bf16_t* __restrict__ a1, const bf16_t* __restrict__ a2, size_t a_step,
                                              const bf16_t* __restrict__ src, const long long* src_off, int K, bool active,
-                                             bf16_t* xt, f32x4 (&acc1)[RB], f32x4 (&acc2)[RB]) {
+                                             bf16_t* xt, f32x4 (&acc1)[NB][RB], f32x4 (&acc2)[NB][RB]) {
     const int lane = threadIdx.x % 64, r = lane % 16, c = lane / 16;
     const int kblocks = (K + 127) / 128;
     for (int kb = 0; kb < kblocks; ++kb) {
@@ -104,15 +106,21 @@ __device__ __forceinline__ void tile_product(const bf16_t* __restrict__ a1, cons
         if (!active) continue;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            const Frag f1 = frag_load(a1 + (size_t)kb * 2048 + j * 512);
-            Frag f2;
-            if (GATED) f2 = frag_load(a2 + (size_t)kb * 2048 + j * 512);
+            Frag f1[NB], f2[NB];
+#pragma unroll
+            for (int i = 0; i < NB; ++i) {
+                f1[i] = frag_load(a1 + i * a_step + (size_t)kb * 2048 + j * 512);
+                if (GATED) f2[i] = frag_load(a2 + i * a_step + (size_t)kb * 2048 + j * 512);
+            }
 #pragma unroll
             for (int b = 0; b < RB; ++b) {
                 Frag fx;
                 fx.u = *reinterpret_cast<const uint4*>(xt + (b * 16 + r) * XT_STRIDE + c * 32 + j * 8);
-                acc1[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f1.v, fx.v, acc1[b], 0, 0, 0);
-                if (GATED) acc2[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f2.v, fx.v, acc2[b], 0, 0, 0);
+#pragma unroll
+                for (int i = 0; i < NB; ++i) {
+                    acc1[i][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f1[i].v, fx.v, acc1[i][b], 0, 0, 0);
+                    if (GATED) acc2[i][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f2[i].v, fx.v, acc2[i][b], 0, 0, 0);
+                }
             }
         }
     }
@@ -134,7 +142,7 @@ __global__ void __launch_bounds__(256) moe_gate_up_kernel(const bf16_t* __restri
     if (tile >= *num_tiles) return;                   // (the whole workgroup)
     const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
     const int r = lane % 16, c = lane / 16;
-    const int nb = blockIdx.x * 4 + wave;             // the wave's block of 16 hidden units
+    const int nb = (blockIdx.x * 4 + wave) * NB;      // the wave's first block of 16 hidden units
     const int nblocks = (ff + 15) / 16, kblocks = (D + 127) / 128;
     const bool active = nb < nblocks;
     const int e = tile_expert[tile];
@@ -142,21 +150,29 @@ __global__ void __launch_bounds__(256) moe_gate_up_kernel(const bf16_t* __restri
         const int p = order[tile * 16 * RB + i];
         src_off[i] = p >= 0 ? (long long)(p / top) * D : -1;
     }
+    // (a block past the last reads the one before it again and stores nothing)
+    const size_t a_step = nb + 1 < nblocks ? (size_t)kblocks * 2048 : 0;
     const size_t block0 = ((size_t)e * nblocks + (active ? nb : 0)) * kblocks * 2048 + lane * 8;
-    f32x4 ag[RB], au[RB];
+    f32x4 ag[NB][RB], au[NB][RB];
 #pragma unroll
-    for (int b = 0; b < RB; ++b) ag[b] = au[b] = (f32x4){0.f, 0.f, 0.f, 0.f};
-    tile_product<RB, true>(gate_t + block0, up_t + block0, x, src_off, D, active, xt, ag, au);
+    for (int i = 0; i < NB; ++i)
+#pragma unroll
+        for (int b = 0; b < RB; ++b) ag[i][b] = au[i][b] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    tile_product<RB, true>(gate_t + block0, up_t + block0, a_step, x, src_off, D, active, xt, ag, au);
     if (!active) return;
-    // the lane holds hidden units nb * 16 + 4 c .. + 4 of the slots 16 b + r
-    const int n0 = nb * 16 + c * 4;
+    // the lane holds hidden units (nb + i) * 16 + 4 c .. + 4 of the slots 16 b + r
 #pragma unroll
-    for (int b = 0; b < RB; ++b) {
-        if (src_off[b * 16 + r] < 0) continue;
-        float h[4];
+    for (int i = 0; i < NB; ++i) {
+        const int n0 = (nb + i) * 16 + c * 4;
+        if (nb + i >= nblocks) continue;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) h[i] = grouped_silu(ag[b][i]) * au[b][i];
-        store4(hid + (size_t)((tile * RB + b) * 16 + r) * ff + n0, h, ff - n0, ff % 4 == 0);
+        for (int b = 0; b < RB; ++b) {
+            if (src_off[b * 16 + r] < 0) continue;
+            float h[4];
+#pragma unroll
+            for (int v = 0; v < 4; ++v) h[v] = grouped_silu(ag[i][b][v]) * au[i][b][v];
+            store4(hid + (size_t)((tile * RB + b) * 16 + r) * ff + n0, h, ff - n0, ff % 4 == 0);
+        }
     }
 }
 
@@ -173,7 +189,7 @@ __global__ void __launch_bounds__(256) moe_down_grouped_kernel(const bf16_t* __r
     if (tile >= *num_tiles) return;
     const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
     const int r = lane % 16, c = lane / 16;
-    const int nb = blockIdx.x * 4 + wave;             // the wave's block of 16 output columns
+    const int nb = (blockIdx.x * 4 + wave) * NB;      // the wave's first block of 16 output columns
     const int nblocks = (D + 15) / 16, kblocks = (ff + 127) / 128;
     const bool active = nb < nblocks;
     const int e = tile_expert[tile];
@@ -181,18 +197,25 @@ __global__ void __launch_bounds__(256) moe_down_grouped_kernel(const bf16_t* __r
         const int slot = tile * 16 * RB + i;
         src_off[i] = order[slot] >= 0 ? (long long)slot * ff : -1;
     }
+    const size_t a_step = nb + 1 < nblocks ? (size_t)kblocks * 2048 : 0;
     const bf16_t* wd = down_t + ((size_t)e * nblocks + (active ? nb : 0)) * kblocks * 2048 + lane * 8;
-    f32x4 acc[RB], unused[RB];
+    f32x4 acc[NB][RB], unused[NB][RB];
 #pragma unroll
-    for (int b = 0; b < RB; ++b) acc[b] = (f32x4){0.f, 0.f, 0.f, 0.f};
-    tile_product<RB, false>(wd, nullptr, hid, src_off, ff, active, xt, acc, unused);
+    for (int i = 0; i < NB; ++i)
+#pragma unroll
+        for (int b = 0; b < RB; ++b) acc[i][b] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    tile_product<RB, false>(wd, nullptr, a_step, hid, src_off, ff, active, xt, acc, unused);
     if (!active) return;
-    const int n0 = nb * 16 + c * 4;
 #pragma unroll
-    for (int b = 0; b < RB; ++b) {
-        if (src_off[b * 16 + r] < 0) continue;
-        const float v[4] = {acc[b][0], acc[b][1], acc[b][2], acc[b][3]};
-        store4(part + (size_t)((tile * RB + b) * 16 + r) * D + n0, v, D - n0, D % 4 == 0);
+    for (int i = 0; i < NB; ++i) {
+        const int n0 = (nb + i) * 16 + c * 4;
+        if (nb + i >= nblocks) continue;
+#pragma unroll
+        for (int b = 0; b < RB; ++b) {
+            if (src_off[b * 16 + r] < 0) continue;
+            const float v[4] = {acc[i][b][0], acc[i][b][1], acc[i][b][2], acc[i][b][3]};
+            store4(part + (size_t)((tile * RB + b) * 16 + r) * D + n0, v, D - n0, D % 4 == 0);
+        }
     }
 }
 
@@ -241,7 +264,7 @@ extern "C" int tli_moe_grouped_bf16(const void* x, const int* ids, const float* 
     hipStream_t s = (hipStream_t)stream;
     hipLaunchKernelGGL(moe_sort_kernel, dim3(1), dim3(1024), 0, s, ids, (int)pairs, E, RT, (int)tiles_max, order, pos,
                        tile_expert, num_tiles);
-    const dim3 g1((ff + 63) / 64, (unsigned)tiles_max), g2((D + 63) / 64, (unsigned)tiles_max);
+    const dim3 g1((ff + 64 * NB - 1) / (64 * NB), (unsigned)tiles_max), g2((D + 64 * NB - 1) / (64 * NB), (unsigned)tiles_max);
 #define TLI_GROUPED(RB)                                                                                              \
     hipLaunchKernelGGL((moe_gate_up_kernel<RB>), g1, dim3(256), 0, s, (const bf16_t*)x, order, tile_expert, num_tiles, \
                        (const bf16_t*)gate_t, (const bf16_t*)up_t, (bf16_t*)hid, top, D, ff);                        \
