@@ -152,6 +152,9 @@ class CpuOps:
     def check_delta_sizes(self, heads, kv_heads, dk, dv, taps):
         pass
 
+    def delta_state_shape(self, heads, dk, dv):
+        return (heads, dk, dv)
+
     def delta_rule(self, proj, gates, conv, a_log, dt_bias, kept, state, step, heads, kv_heads, dk, dv, taps):
         T = step.num_rows
         qd, vd = kv_heads * dk, heads * dv

@@ -130,7 +130,7 @@ def test_delta_rule_kernels_in_portions_and_decoding(ops, dtype, H, G, dk, dv, t
     raw = {k: torch.randn(n, ld, generator=g) for k, n in lengths.items()}
     gates = {k: torch.randn(n, 2 * H, generator=g) for k, n in lengths.items()}
     want = {k: _plain_delta_core(raw[k], gates[k], conv, a_log, dt_bias, norm_w, 1e-5, H, G, dk, dv, dt) for k in lengths}
-    S = torch.full((3, H, dk, dv), 7.0, dtype=torch.float32, device="cuda")           # slots are never cleared
+    S = torch.full((3,) + tuple(ops.delta_state_shape(H, dk, dv)), 7.0, dtype=torch.float32, device="cuda")   # slots are never cleared
     kept = torch.full((3, max(taps - 1, 1), C), 5.0, dtype=dt, device="cuda") if taps > 1 else None
     slot = {"a": 0, "b": 1, "c": 2, "d": 1}                                       # d takes b's slot when b is done
     plan = [{"a": 3, "b": 9}, {"a": 1, "c": 2}, {"a": 40, "c": 1, "d": 1}, {"c": 1, "d": 2, "a": 2}, {"d": 27, "c": 43, "a": 15}]

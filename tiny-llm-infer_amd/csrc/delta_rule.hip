@@ -9,8 +9,8 @@
 //   recurrence:  S <- decay S;  u = beta (v' - S^T k');  S <- S + k' u^T;  o = S^T q'
 //   gated norm:  y = o / sqrt(mean(o^2) + eps) * w * silu(gate)         per head, over dv
 //
-// S is float32 [dk, dv] a head and lives in a slot of per-request state, as do the last taps - 1 raw
-// rows that the convolution reads.  A sequence that starts at position 0 has no history: its slot is
+// S is float32 [dk, dv] a head and lives in a slot of per-request state (in the order the recurrence
+// kernel's lanes hold it, see there), as do the last taps - 1 raw rows that the convolution reads.  A sequence that starts at position 0 has no history: its slot is
 // not read.  Everything after the projections is float32.
 //
 // The recurrence walks a sequence's rows one after the other.  Columns of S are independent, so a
@@ -150,13 +150,13 @@ __global__ __launch_bounds__(256) void delta_recurrence_kernel(
     const int kvh = head / (H / G);
     const int r0 = row_start[seq], r1 = row_start[seq + 1];
     const bool fresh = seq_start[seq] == 0;
-    float* mine = state + ((size_t)slots[seq] * H + head) * dk * dv;
+    // The state of a slot: [head][block of 16 columns][r][column][part], element i = part + 16 r of a column: a
+    // wave's 64 lanes read and write 64 floats in a row.  Elements past dk and columns past dv exist there too
+    // (they stay 0: their k is 0, and the v of a column past dv is read as 0).
+    float* mine = state + ((((size_t)slots[seq] * H + head) * gridDim.x + blockIdx.x) * RPT * DELTA_COLS + local) * DELTA_LANES + part;
     float S[RPT];
 #pragma unroll
-    for (int r = 0; r < RPT; ++r) {
-        const int i = part + DELTA_LANES * r;
-        S[r] = (!fresh && i < dk) ? mine[(size_t)i * dv + col] : 0.f;
-    }
+    for (int r = 0; r < RPT; ++r) S[r] = fresh ? 0.f : mine[(size_t)r * DELTA_COLS * DELTA_LANES];
     const size_t qd = (size_t)G * dk, vd = (size_t)H * dv;
     float pk[NK], pq[NK], pv[NV], ps = 0.f;
     auto fetch = [&](int c0) {                   // the chunk that starts at row c0, into registers
@@ -225,13 +225,8 @@ __global__ __launch_bounds__(256) void delta_recurrence_kernel(
             if (part == 0 && live) out[(size_t)(c0 + t) * vd + (size_t)head * dv + col] = fmaf(c0q, u, g0 * s2);
         }
     }
-    if (live) {
 #pragma unroll
-        for (int r = 0; r < RPT; ++r) {
-            const int i = part + DELTA_LANES * r;
-            if (i < dk) mine[(size_t)i * dv + col] = S[r];
-        }
-    }
+    for (int r = 0; r < RPT; ++r) mine[(size_t)r * DELTA_COLS * DELTA_LANES] = S[r];
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -298,6 +293,13 @@ extern "C" int tli_delta_prepare(const void* proj, int ld, const float* conv_w, 
         return tli_fail("delta_prepare: unknown dtype %d", dtype);
     }
     return tli_check_launch("delta_prepare");
+}
+
+// Floats of state a head: columns in blocks of 16, key elements padded to 16 * RPT (RPT = 1, 2, 4, 8 or 16).
+extern "C" int tli_delta_state_floats(int dk, int dv) {
+    if (dk <= 0 || dv <= 0 || dk > DELTA_MAX_DK) return 0;
+    const int rpt = dk <= 16 ? 1 : dk <= 32 ? 2 : dk <= 64 ? 4 : dk <= 128 ? 8 : 16;
+    return ((dv + DELTA_COLS - 1) / DELTA_COLS) * rpt * DELTA_COLS * DELTA_LANES;
 }
 
 extern "C" int tli_delta_recurrence(const float* qn, const float* kn, const float* vc, const float* beta,

@@ -106,6 +106,7 @@ def load_library():
         "tli_add_layernorm": [P, P, P, P, P, P, P, P, I, I, I, F, I, P],
         "tli_delta_prepare": [P, I, P, P, P, P, P, P, P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, P],
         "tli_delta_recurrence": [P, P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, P],
+        "tli_delta_state_floats": [I, I],
         "tli_gated_rmsnorm": [P, P, I, P, P, I, I, I, F, I, P],
         "tli_moe_route": [P, I, P, P, P, I, I, I, I, I, F, I, P],
         "tli_moe_experts": [P, P, P, P, P, P, P, P, P, I, I, I, I, I, P],
@@ -1080,11 +1081,19 @@ class HipOps:
         if (2 * kv_heads * dk + heads * dv) * 4 > 64 * 1024:
             raise KernelError("the channels of q, k and v of a row do not fit a workgroup's memory")
 
+    def delta_state_shape(self, heads: int, dk: int, dv: int):
+        """The shape of one request's recurrent state (float32).  The recurrence kernel keeps a head's [dk, dv]
+        matrix in the order its lanes hold it, padded to whole blocks, so that it reads and writes it in runs."""
+        n = int(self.lib.tli_delta_state_floats(dk, dv))
+        if n <= 0:
+            raise KernelError(f"a state of {dk} x {dv} a head is not supported")
+        return (heads, n)
+
     def delta_rule(self, proj, gates, conv, a_log, dt_bias, kept, state, step, heads, kv_heads, dk, dv, taps):
         """From the raw projections ``proj`` [T, >= channels] (q, k, v first) and ``gates`` (float32 [T, 2 H]:
         b, then a) to the heads' outputs of the recurrence, float32 [T, H dv].  ``conv``: float32 [taps,
-        channels], oldest tap first; ``kept`` [slots, taps - 1, channels] and ``state`` (float32 [slots, H,
-        dk, dv]) are the sequences' state, read (unless a sequence starts at position 0) and replaced."""
+        channels], oldest tap first; ``kept`` [slots, taps - 1, channels] and ``state`` (float32 [slots,
+        *delta_state_shape]) are the sequences' state, read (unless a sequence starts at position 0) and replaced."""
         T = step.num_rows
         self.check_delta_sizes(heads, kv_heads, dk, dv, taps)
         qd, vd = kv_heads * dk, heads * dv
@@ -1096,7 +1105,7 @@ class HipOps:
         self._want(conv, "convolution weights", torch.float32, (taps, C))
         self._want(a_log, "A_log", torch.float32, (heads,))
         self._want(dt_bias, "dt_bias", torch.float32, (heads,))
-        self._want(state, "recurrent state", torch.float32, (state.shape[0], heads, dk, dv))
+        self._want(state, "recurrent state", torch.float32, (state.shape[0],) + self.delta_state_shape(heads, dk, dv))
         slots = state.shape[0]
         if taps > 1:
             if kept is None:

@@ -79,7 +79,8 @@ class GatedDeltaRule(Mixer):
         self.w_o = as_matrix(weights[n["o"]], env)
 
     def state_need(self):
-        needs = {"S": StateNeed((self.heads, self.dk, self.dv), torch.float32)}
+        # (the kernel library says in which order, and padded how, it keeps a head's matrix)
+        needs = {"S": StateNeed(tuple(self.env.ops.delta_state_shape(self.heads, self.dk, self.dv)), torch.float32)}
         if self.taps > 1:
             needs["conv"] = StateNeed((self.taps - 1, self.channels), None)
         return needs
