@@ -91,6 +91,21 @@ __device__ __forceinline__ void tile_product(const bf16_t* __restrict__ a1, cons
                                              bf16_t* xt, f32x4 (&acc1)[NB][RB], f32x4 (&acc2)[NB][RB]) {
     const int lane = threadIdx.x % 64, r = lane % 16, c = lane / 16;
     const int kblocks = (K + 127) / 128;
+    // Small tiles (decode steps) are few workgroups that stream whole matrices: the fragments of A of the block
+    // of k after the current one are asked for before the current one's products run.  Large tiles have their
+    // registers full of sums and many workgroups in flight instead.
+    constexpr bool AHEAD = RB <= 2;
+    Frag n1[4][NB], n2[4][NB];
+    auto fetch_a = [&](int kb) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int i = 0; i < NB; ++i) {
+                n1[j][i] = frag_load(a1 + i * a_step + (size_t)kb * 2048 + j * 512);
+                if (GATED) n2[j][i] = frag_load(a2 + i * a_step + (size_t)kb * 2048 + j * 512);
+            }
+    };
+    if (AHEAD && active) fetch_a(0);
     for (int kb = 0; kb < kblocks; ++kb) {
         __syncthreads();
 #pragma unroll
@@ -104,13 +119,25 @@ __device__ __forceinline__ void tile_product(const bf16_t* __restrict__ a1, cons
         }
         __syncthreads();
         if (!active) continue;
+        Frag f1[4][NB], f2[4][NB];
+        if (AHEAD) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int i = 0; i < NB; ++i) {
+                    f1[j][i] = n1[j][i];
+                    if (GATED) f2[j][i] = n2[j][i];
+                }
+            fetch_a(min(kb + 1, kblocks - 1));           // (the last block once more rather than a branch around loads)
+        }
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            Frag f1[NB], f2[NB];
+            if (!AHEAD) {
 #pragma unroll
-            for (int i = 0; i < NB; ++i) {
-                f1[i] = frag_load(a1 + i * a_step + (size_t)kb * 2048 + j * 512);
-                if (GATED) f2[i] = frag_load(a2 + i * a_step + (size_t)kb * 2048 + j * 512);
+                for (int i = 0; i < NB; ++i) {
+                    f1[j][i] = frag_load(a1 + i * a_step + (size_t)kb * 2048 + j * 512);
+                    if (GATED) f2[j][i] = frag_load(a2 + i * a_step + (size_t)kb * 2048 + j * 512);
+                }
             }
 #pragma unroll
             for (int b = 0; b < RB; ++b) {
@@ -118,8 +145,8 @@ __device__ __forceinline__ void tile_product(const bf16_t* __restrict__ a1, cons
                 fx.u = *reinterpret_cast<const uint4*>(xt + (b * 16 + r) * XT_STRIDE + c * 32 + j * 8);
 #pragma unroll
                 for (int i = 0; i < NB; ++i) {
-                    acc1[i][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f1[i].v, fx.v, acc1[i][b], 0, 0, 0);
-                    if (GATED) acc2[i][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f2[i].v, fx.v, acc2[i][b], 0, 0, 0);
+                    acc1[i][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f1[j][i].v, fx.v, acc1[i][b], 0, 0, 0);
+                    if (GATED) acc2[i][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f2[j][i].v, fx.v, acc2[i][b], 0, 0, 0);
                 }
             }
         }
