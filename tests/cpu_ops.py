@@ -152,11 +152,16 @@ class CpuOps:
     def check_delta_sizes(self, heads, kv_heads, dk, dv, taps):
         pass
 
+    def small_product(self, x, w_rows):
+        return x.to(torch.float32) @ w_rows.to(torch.float32).t(), False
+
     def delta_state_shape(self, heads, dk, dv):
         return (heads, dk, dv)
 
-    def delta_rule(self, proj, gates, conv, a_log, dt_bias, kept, state, step, heads, kv_heads, dk, dv, taps):
+    def delta_rule(self, proj, gates, conv, a_log, dt_bias, kept, state, step, heads, kv_heads, dk, dv, taps,
+                   gates_transposed=False):
         T = step.num_rows
+        gates = gates.t() if gates_transposed else gates
         qd, vd = kv_heads * dk, heads * dv
         C = 2 * qd + vd
         raw = proj[:, :C].to(torch.float32)
@@ -204,7 +209,8 @@ class CpuOps:
     def pack_experts(self, w_gate_up, w_down):
         return None
 
-    def route_experts(self, z, experts, top, groups, keep, scale, has_shared):
+    def route_experts(self, z, experts, top, groups, keep, scale, has_shared, transposed=False):
+        z = z.t() if transposed else z
         T = z.shape[0]
         s = torch.sigmoid(z[:, :experts])
         per = experts // groups

@@ -141,7 +141,9 @@ def test_delta_rule_kernels_in_portions_and_decoding(ops, dtype, H, G, dk, dv, t
         view = _view([at[k] for k in keys], [portions[k] for k in keys], [slot[k] for k in keys])
         proj = torch.cat([raw[k][at[k]:at[k] + portions[k]] for k in keys]).to(dt).cuda()
         ba = torch.cat([gates[k][at[k]:at[k] + portions[k]] for k in keys]).cuda()
-        o = ops.delta_rule(proj, ba, conv.t().contiguous().cuda(), a_log.cuda(), dt_bias.cuda(), kept, S, view, H, G, dk, dv, taps)
+        turned = len(keys) % 2 == 1                       # b and a as [2 H, rows] in every other step
+        o = ops.delta_rule(proj, ba.t().contiguous() if turned else ba, conv.t().contiguous().cuda(), a_log.cuda(),
+                           dt_bias.cuda(), kept, S, view, H, G, dk, dv, taps, gates_transposed=turned)
         y = ops.gated_rmsnorm(o, proj, C, norm_w.cuda(), 1e-5, H, dv, dt)
         r = 0
         for k in keys:
@@ -167,6 +169,18 @@ def test_router_choice_and_weights(ops, E, top, groups, keep):
     _close(gate, torch.sigmoid(z[:, E].double()), 1e-6, "shared gate")
     ids2, wts2, none = ops.route_experts(z[:, :E].contiguous().cuda(), E, top, groups, keep, 2.5, False)
     assert none is None and torch.equal(ids2, ids) and torch.equal(wts2, wts)
+    ids3, wts3, gate3 = ops.route_experts(z.t().contiguous().cuda(), E, top, groups, keep, 2.5, True, transposed=True)
+    assert torch.equal(ids3, ids) and torch.equal(wts3, wts) and torch.equal(gate3, gate)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("T, N, K", [(1, 9, 64), (5, 3, 100), (64, 17, 256), (300, 70, 128), (2048, 33, 512)])
+def test_product_with_a_matrix_of_few_rows(ops, dtype, T, N, K):
+    g = torch.Generator().manual_seed(T + N)
+    x, w = torch.randn(T, K, generator=g).to(DTYPES[dtype]), torch.randn(N, K, generator=g).to(DTYPES[dtype])
+    y, transposed = ops.small_product(x.cuda(), w.cuda())
+    assert y.dtype == torch.float32 and transposed == (dtype == "bfloat16" and K % 8 == 0)
+    _close(y.t() if transposed else y, x.double() @ w.double().t(), 2e-6, "product")
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16", "bfloat16-plain", "bfloat16-tiles-of-16", "bfloat16-tiles-of-64", "bfloat16-tiles-of-128"])

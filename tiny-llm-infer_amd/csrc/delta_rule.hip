@@ -26,8 +26,8 @@ __device__ __forceinline__ float silu_f(float z) { return z / (1.0f + expf(-z));
 // ---------------------------------------------------------------------------------------------
 template <typename T>
 __global__ void delta_prepare_kernel(const T* __restrict__ proj, int ld, const float* __restrict__ conv_w,
-                                     const T* __restrict__ kept, const float* __restrict__ ba,
-                                     const float* __restrict__ a_log, const float* __restrict__ dt_bias,
+                                     const T* __restrict__ kept, const float* __restrict__ ba, long long ba_row,
+                                     long long ba_col, const float* __restrict__ a_log, const float* __restrict__ dt_bias,
                                      const int* __restrict__ positions, const int* __restrict__ seq_of_row,
                                      const int* __restrict__ row_start, const int* __restrict__ slots,
                                      float* __restrict__ qn, float* __restrict__ kn, float* __restrict__ vc,
@@ -72,7 +72,8 @@ __global__ void delta_prepare_kernel(const T* __restrict__ proj, int ld, const f
     for (int i = threadIdx.x; i < H * dv; i += blockDim.x) vc[(size_t)r * H * dv + i] = buf[2 * qd + i];
     if (threadIdx.x < H) {
         const int h = threadIdx.x;
-        const float b = ba[(size_t)r * 2 * H + h], a = ba[(size_t)r * 2 * H + H + h] + dt_bias[h];
+        const float b = ba[(size_t)r * ba_row + (size_t)h * ba_col];
+        const float a = ba[(size_t)r * ba_row + (size_t)(H + h) * ba_col] + dt_bias[h];
         beta[(size_t)r * H + h] = 1.0f / (1.0f + expf(-b));
         const float sp = fmaxf(a, 0.f) + log1pf(expf(-fabsf(a)));
         decay[(size_t)r * H + h] = expf(-expf(a_log[h]) * sp);
@@ -258,10 +259,10 @@ __global__ void gated_rmsnorm_kernel(const float* __restrict__ o, const T* __res
 
 // proj: [T, ld] raw projections, channels q (G dk), k (G dk), v (H dv) first; conv_w: float32
 // [taps, channels], oldest tap first; kept: [slots, taps - 1, channels] or null for one tap;
-// ba: float32 [T, 2 H], b then a.  Outputs are float32: qn, kn [T, G dk], vc [T, H dv], beta, decay
+// ba: float32, b then a: number n of row t at t * ba_row + n * ba_col.  Outputs are float32: qn, kn [T, G dk], vc [T, H dv], beta, decay
 // [T, H], qk [T, G].  `keep`: also move the kept rows on (after every row was read).
 extern "C" int tli_delta_prepare(const void* proj, int ld, const float* conv_w, void* kept, const float* ba,
-                                 const float* a_log, const float* dt_bias, const int* positions,
+                                 long long ba_row, long long ba_col, const float* a_log, const float* dt_bias, const int* positions,
                                  const int* seq_of_row, const int* row_start, const int* seq_start, const int* slots,
                                  float* qn, float* kn, float* vc, float* beta, float* decay, float* qk, int T,
                                  int seqs, int H, int G, int dk, int dv, int taps, int dtype, void* stream) {
@@ -277,14 +278,14 @@ extern "C" int tli_delta_prepare(const void* proj, int ld, const float* conv_w, 
     hipStream_t s = (hipStream_t)stream;
     if (dtype == TLI_F32) {
         hipLaunchKernelGGL((delta_prepare_kernel<float>), dim3(T), dim3(256), lds, s, (const float*)proj, ld, conv_w,
-                           (const float*)kept, ba, a_log, dt_bias, positions, seq_of_row, row_start, slots, qn, kn, vc,
+                           (const float*)kept, ba, ba_row, ba_col, a_log, dt_bias, positions, seq_of_row, row_start, slots, qn, kn, vc,
                            beta, decay, qk, H, G, dk, dv, taps);
         if (taps > 1)
             hipLaunchKernelGGL((delta_conv_keep_kernel<float>), dim3((C + 255) / 256, seqs), dim3(256), 0, s,
                                (const float*)proj, ld, (float*)kept, row_start, seq_start, slots, C, taps);
     } else if (dtype == TLI_BF16) {
         hipLaunchKernelGGL((delta_prepare_kernel<bf16_t>), dim3(T), dim3(256), lds, s, (const bf16_t*)proj, ld, conv_w,
-                           (const bf16_t*)kept, ba, a_log, dt_bias, positions, seq_of_row, row_start, slots, qn, kn,
+                           (const bf16_t*)kept, ba, ba_row, ba_col, a_log, dt_bias, positions, seq_of_row, row_start, slots, qn, kn,
                            vc, beta, decay, qk, H, G, dk, dv, taps);
         if (taps > 1)
             hipLaunchKernelGGL((delta_conv_keep_kernel<bf16_t>), dim3((C + 255) / 256, seqs), dim3(256), 0, s,

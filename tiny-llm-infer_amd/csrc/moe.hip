@@ -17,16 +17,16 @@
 
 #define MOE_MAX_TOP 32
 
-__global__ void moe_route_kernel(const float* __restrict__ z, int ldz, int* __restrict__ ids,
+__global__ void moe_route_kernel(const float* __restrict__ z, long long z_row, long long z_col, int* __restrict__ ids,
                                  float* __restrict__ weights, float* __restrict__ shared_gate, int T, int E,
                                  int top, int groups, int keep, float scale, int has_shared) {
     extern __shared__ float sig[];                 // [threads][E + 1]: a row's scores (odd stride: no bank conflicts)
     const int t = blockIdx.x * blockDim.x + threadIdx.x;
     if (t >= T) return;
     float* s = sig + (size_t)threadIdx.x * (E + 1);
-    const float* zr = z + (size_t)t * ldz;
-    for (int e = 0; e < E; ++e) s[e] = 1.0f / (1.0f + expf(-zr[e]));
-    if (has_shared) shared_gate[t] = 1.0f / (1.0f + expf(-zr[E]));
+    const float* zr = z + (size_t)t * z_row;              // logit e of row t lies at t * z_row + e * z_col
+    for (int e = 0; e < E; ++e) s[e] = 1.0f / (1.0f + expf(-zr[(size_t)e * z_col]));
+    if (has_shared) shared_gate[t] = 1.0f / (1.0f + expf(-zr[(size_t)E * z_col]));
     const int per = E / groups;
     // the `keep` best groups, as a bit a group (groups <= 64)
     unsigned long long open = 0ull;
@@ -127,18 +127,19 @@ __global__ void moe_down_kernel(const T* __restrict__ hid, const int* __restrict
     }
 }
 
-extern "C" int tli_moe_route(const float* z, int ldz, int* ids, float* weights, float* shared_gate, int T, int E,
-                             int top, int groups, int keep, float scale, int has_shared, void* stream) {
+extern "C" int tli_moe_route(const float* z, long long z_row, long long z_col, int* ids, float* weights,
+                             float* shared_gate, int T, int E, int top, int groups, int keep, float scale, int has_shared,
+                             void* stream) {
     if (T <= 0) return 0;
     if (E <= 0 || top <= 0 || top > E || top > MOE_MAX_TOP || groups <= 0 || groups > 64 || E % groups || keep <= 0 ||
-        keep > groups || (long long)keep * (E / groups) < top || ldz < E + (has_shared ? 1 : 0))
+        keep > groups || (long long)keep * (E / groups) < top || z_row <= 0 || z_col <= 0)
         return tli_fail("moe_route: bad sizes (experts %d, top %d (at most %d), groups %d (at most 64), keep %d)", E,
                         top, MOE_MAX_TOP, groups, keep);
     if (E > 2048) return tli_fail("moe_route: at most 2048 experts, got %d", E);
     int threads = 64;
     while (threads > 1 && (size_t)threads * (E + 1) * sizeof(float) > 48 * 1024) threads /= 2;
     hipLaunchKernelGGL(moe_route_kernel, dim3((T + threads - 1) / threads), dim3(threads),
-                       (size_t)threads * (E + 1) * sizeof(float), (hipStream_t)stream, z, ldz, ids, weights, shared_gate,
+                       (size_t)threads * (E + 1) * sizeof(float), (hipStream_t)stream, z, z_row, z_col, ids, weights, shared_gate,
                        T, E, top, groups, keep, scale, has_shared);
     return tli_check_launch("moe_route");
 }

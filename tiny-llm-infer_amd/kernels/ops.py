@@ -104,11 +104,12 @@ def load_library():
         "tli_attention_biased_plain": [P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, P, P, P, I, I, I, P],
         "tli_attention_biased_mfma_bf16": [P, P, P, P, P, P, I, I, I, P, I, I, I, I, I, I, F, P, P, P, I, I, I, P],
         "tli_add_layernorm": [P, P, P, P, P, P, P, P, I, I, I, F, I, P],
-        "tli_delta_prepare": [P, I, P, P, P, P, P, P, P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, P],
+        "tli_delta_prepare": [P, I, P, P, P, ctypes.c_longlong, ctypes.c_longlong, P, P, P, P, P, P, P, P, P, P, P, P, P,
+                              I, I, I, I, I, I, I, I, P],
         "tli_delta_recurrence": [P, P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, P],
         "tli_delta_state_floats": [I, I],
         "tli_gated_rmsnorm": [P, P, I, P, P, I, I, I, F, I, P],
-        "tli_moe_route": [P, I, P, P, P, I, I, I, I, I, F, I, P],
+        "tli_moe_route": [P, ctypes.c_longlong, ctypes.c_longlong, P, P, P, I, I, I, I, I, F, I, P],
         "tli_moe_experts": [P, P, P, P, P, P, P, P, P, I, I, I, I, I, P],
         "tli_moe_grouped_tile": [I, I],
         "tli_moe_grouped_bf16": [P, P, P, P, P, P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, P],
@@ -1081,6 +1082,24 @@ class HipOps:
         if (2 * kv_heads * dk + heads * dv) * 4 > 64 * 1024:
             raise KernelError("the channels of q, k and v of a row do not fit a workgroup's memory")
 
+    def small_product(self, x: torch.Tensor, w_rows: torch.Tensor):
+        """x W^T in float32 for a matrix of few rows (a router, a few numbers a head): returns (y, transposed).
+        In a bfloat16 run the roles are swapped, the few rows of W being the rows of a product that streams x as
+        its matrix: one launch for any number of rows of x, and y comes out as [rows of W, rows of x]
+        (``transposed``); otherwise y is [rows of x, rows of W] from the ordinary product."""
+        M, K = x.shape
+        N = w_rows.shape[0]
+        self._want(x, "product input")
+        self._want(w_rows, "matrix of few rows", x.dtype, (N, K))
+        if x.dtype != torch.bfloat16 or K % 8 or self.plain_products or M == 0:
+            return self.linear_plain(x, w_rows, torch.float32), False
+        y = torch.empty((N, M), dtype=torch.float32, device=self.device)
+        for n0 in range(0, N, self.SKINNY_ROWS):
+            n1 = min(N, n0 + self.SKINNY_ROWS)
+            self._call(self.lib.tli_gemm_skinny_bf16, w_rows[n0:n1].data_ptr(), x.data_ptr(), y[n0:n1].data_ptr(), n1 - n0, M, K,
+                       F32, 0, 0, self._stream())
+        return y, True
+
     def delta_state_shape(self, heads: int, dk: int, dv: int):
         """The shape of one request's recurrent state (float32).  The recurrence kernel keeps a head's [dk, dv]
         matrix in the order its lanes hold it, padded to whole blocks, so that it reads and writes it in runs."""
@@ -1089,9 +1108,10 @@ class HipOps:
             raise KernelError(f"a state of {dk} x {dv} a head is not supported")
         return (heads, n)
 
-    def delta_rule(self, proj, gates, conv, a_log, dt_bias, kept, state, step, heads, kv_heads, dk, dv, taps):
+    def delta_rule(self, proj, gates, conv, a_log, dt_bias, kept, state, step, heads, kv_heads, dk, dv, taps,
+                   gates_transposed=False):
         """From the raw projections ``proj`` [T, >= channels] (q, k, v first) and ``gates`` (float32 [T, 2 H]:
-        b, then a) to the heads' outputs of the recurrence, float32 [T, H dv].  ``conv``: float32 [taps,
+        b, then a; [2 H, T] with ``gates_transposed``) to the heads' outputs of the recurrence, float32 [T, H dv].  ``conv``: float32 [taps,
         channels], oldest tap first; ``kept`` [slots, taps - 1, channels] and ``state`` (float32 [slots,
         *delta_state_shape]) are the sequences' state, read (unless a sequence starts at position 0) and replaced."""
         T = step.num_rows
@@ -1101,7 +1121,8 @@ class HipOps:
         if proj.dim() != 2 or proj.shape[0] != T or proj.shape[1] < C:
             raise KernelError(f"the projections have shape {tuple(proj.shape)}, expected [{T}, >= {C}]")
         self._want(proj, "projections")
-        self._want(gates, "b and a", torch.float32, (T, 2 * heads))
+        self._want(gates, "b and a", torch.float32, (2 * heads, T) if gates_transposed else (T, 2 * heads))
+        ba_row, ba_col = (1, T) if gates_transposed else (2 * heads, 1)
         self._want(conv, "convolution weights", torch.float32, (taps, C))
         self._want(a_log, "A_log", torch.float32, (heads,))
         self._want(dt_bias, "dt_bias", torch.float32, (heads,))
@@ -1118,7 +1139,7 @@ class HipOps:
         vc, out = torch.empty((T, vd), **f32), torch.empty((T, vd), **f32)
         beta, decay, qk = torch.empty((T, heads), **f32), torch.empty((T, heads), **f32), torch.empty((T, kv_heads), **f32)
         self._call(self.lib.tli_delta_prepare, proj.data_ptr(), proj.shape[1], conv.data_ptr(), _ptr(kept), gates.data_ptr(),
-                   a_log.data_ptr(), dt_bias.data_ptr(), step.positions.data_ptr(), step.seq_of_row.data_ptr(),
+                   ba_row, ba_col, a_log.data_ptr(), dt_bias.data_ptr(), step.positions.data_ptr(), step.seq_of_row.data_ptr(),
                    step.row_start.data_ptr(), step.seq_start.data_ptr(), step.slots.data_ptr(), qn.data_ptr(),
                    kn.data_ptr(), vc.data_ptr(), beta.data_ptr(), decay.data_ptr(), qk.data_ptr(), T, step.num_seqs,
                    heads, kv_heads, dk, dv, taps, _dtype_code(proj.dtype), self._stream())
@@ -1165,15 +1186,17 @@ class HipOps:
                 "down": torch.stack([self.tile_matrix(w_down[e]) for e in range(E)]),
                 "experts": E, "hidden": n, "inter": ff}
 
-    def route_experts(self, z, experts, top, groups, keep, scale, has_shared):
-        """From router logits ``z`` (float32 [T, E (+ 1)]) to the chosen experts (int32 [T, top]), their
+    def route_experts(self, z, experts, top, groups, keep, scale, has_shared, transposed=False):
+        """From router logits ``z`` (float32 [T, E (+ 1)]; [E (+ 1), T] with ``transposed``) to the chosen experts (int32 [T, top]), their
         weights (float32 [T, top]) and, if the last column is a shared expert's gate, its sigmoid [T]."""
-        T = z.shape[0]
-        self._want(z, "router logits", torch.float32, (T, experts + (1 if has_shared else 0)))
+        T = z.shape[1] if transposed else z.shape[0]
+        columns = experts + (1 if has_shared else 0)
+        self._want(z, "router logits", torch.float32, (columns, T) if transposed else (T, columns))
+        z_row, z_col = (1, T) if transposed else (columns, 1)
         ids = torch.empty((T, top), dtype=torch.int32, device=self.device)
         weights = torch.empty((T, top), dtype=torch.float32, device=self.device)
         gate = torch.empty((T,), dtype=torch.float32, device=self.device) if has_shared else None
-        self._call(self.lib.tli_moe_route, z.data_ptr(), z.shape[1], ids.data_ptr(), weights.data_ptr(), _ptr(gate), T,
+        self._call(self.lib.tli_moe_route, z.data_ptr(), z_row, z_col, ids.data_ptr(), weights.data_ptr(), _ptr(gate), T,
                    experts, top, groups, keep, float(scale), 1 if has_shared else 0, self._stream())
         return ids, weights, gate
 

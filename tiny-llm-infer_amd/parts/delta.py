@@ -73,7 +73,7 @@ class GatedDeltaRule(Mixer):
         # one product for everything that stays in the run's type (q, k, v, then the output gate),
         # one for the two numbers a head that the recurrence wants in float32 (b, then a)
         self.w_main = fuse_rows([weights[n[r]] for r in ("q", "k", "v", "gate")], env)
-        self.w_gates = fuse_rows([weights[n["b"]], weights[n["a"]]], env)
+        self.w_gates = torch.cat([weights[n["b"]].to(env.dtype), weights[n["a"]].to(env.dtype)], dim=0).contiguous()   # few rows: kept row-major
         self.conv = f32("q_conv", "k_conv", "v_conv").t().contiguous()      # [taps, channels]: tap by tap
         self.a_log, self.dt_bias, self.norm = f32("a_log"), f32("dt_bias"), f32("norm")
         self.w_o = as_matrix(weights[n["o"]], env)
@@ -92,10 +92,10 @@ class GatedDeltaRule(Mixer):
     def forward(self, x: torch.Tensor, step: StepView):
         ops = self.env.ops
         main = ops.linear(x, self.w_main)
-        gates = ops.linear(x, self.w_gates, out_dtype=torch.float32)
+        gates, transposed = ops.small_product(x, self.w_gates)
         states = step.state
         o = ops.delta_rule(main, gates, self.conv, self.a_log, self.dt_bias, states.get("conv"), states["S"], step,
-                           self.heads, self.kv_heads, self.dk, self.dv, self.taps)
+                           self.heads, self.kv_heads, self.dk, self.dv, self.taps, gates_transposed=transposed)
         y = ops.gated_rmsnorm(o, main, self.channels, self.norm, self.eps, self.heads, self.dv, self.env.dtype)
         return ops.linear(y, self.w_o, deferred=True)
 

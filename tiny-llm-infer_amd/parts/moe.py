@@ -20,7 +20,7 @@ import torch
 
 from ..weights.loader import TensorDecl
 from .base import BuildEnv, FeedForward, StepView, register_part
-from .linear import GatedMatrix, as_matrix, fuse_rows
+from .linear import GatedMatrix, as_matrix
 
 
 class RoutedExperts(FeedForward):
@@ -64,7 +64,7 @@ class RoutedExperts(FeedForward):
         n = self.spec.names
         env.ops.check_expert_sizes(self.experts, self.top, self.groups, self.keep, self.hidden, self.inter)
         rows = [weights[n["router"]]] + ([weights[n["shared_scale"]]] if self.shared_inter is not None else [])
-        self.w_router = fuse_rows(rows, env)
+        self.w_router = torch.cat([r.to(env.dtype) for r in rows], dim=0).contiguous()       # few rows: kept row-major
         # the experts' matrices side by side: [E, 2 ff, hidden] (an expert's gate rows, then its up rows), [E, hidden, ff]
         self.w_gate_up = torch.stack([torch.cat([weights[self._expert(j, "gate")], weights[self._expert(j, "up")]], dim=0)
                                       for j in range(self.experts)]).to(env.dtype).contiguous()
@@ -84,9 +84,9 @@ class RoutedExperts(FeedForward):
 
     def forward(self, x: torch.Tensor, step: StepView):
         ops = self.env.ops
-        z = ops.linear(x, self.w_router, out_dtype=torch.float32)
+        z, transposed = ops.small_product(x, self.w_router)
         ids, weights, shared_gate = ops.route_experts(z, self.experts, self.top, self.groups, self.keep, self.scale,
-                                                      self.shared_inter is not None)
+                                                      self.shared_inter is not None, transposed)
         shared = None
         if self.shared_inter is not None:
             shared = ops.linear(ops.linear_swiglu(x, self.shared_gate_up), self.shared_down)
