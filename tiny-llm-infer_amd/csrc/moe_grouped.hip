@@ -83,9 +83,10 @@ __global__ void __launch_bounds__(1024) moe_sort_kernel(const int* __restrict__ 
 // LDS by all threads together (rows without a pair, and columns past the end, as zeros), then every
 // wave takes its fragments from there.  `src_off`: for each of the tile's rows the offset of its
 // source row, or a negative number.
-#define NB 2                   // blocks of 16 outputs a wave takes: a fragment of B from LDS serves that many products
+// NB: blocks of 16 outputs a wave takes; a fragment of B from LDS serves that many products (of each of the two
+// matrices, if GATED).  Two, but one where gate and up over 128 slots would leave no registers for running ahead.
 
-template <int RB, bool GATED>
+template <int RB, int NB, bool GATED>
 __device__ __forceinline__ void tile_product(const bf16_t* __restrict__ a1, const bf16_t* __restrict__ a2, size_t a_step,
                                              const bf16_t* __restrict__ src, const long long* src_off, int K, bool active,
                                              bf16_t* xt, f32x4 (&acc1)[NB][RB], f32x4 (&acc2)[NB][RB]) {
@@ -105,22 +106,22 @@ __device__ __forceinline__ void tile_product(const bf16_t* __restrict__ a1, cons
                 if (GATED) n2[j][i] = frag_load(a2 + i * a_step + (size_t)kb * 2048 + j * 512);
             }
     };
-    if (AHEAD && active) fetch_a(0);
-    for (int kb = 0; kb < kblocks; ++kb) {
-        __syncthreads();
+    if (AHEAD) {
+        if (active) fetch_a(0);
+        for (int kb = 0; kb < kblocks; ++kb) {
+            __syncthreads();
 #pragma unroll
-        for (int n = 0; n < RB; ++n) {
-            const int id = threadIdx.x + n * 256, row = id / 16, kc = id % 16;
-            const long long off = src_off[row];
-            const int k = kb * 128 + kc * 8;
-            uint4 v = make_uint4(0, 0, 0, 0);
-            if (off >= 0 && k + 8 <= K) v = *reinterpret_cast<const uint4*>(src + off + k);
-            *reinterpret_cast<uint4*>(xt + row * XT_STRIDE + kc * 8) = v;
-        }
-        __syncthreads();
-        if (!active) continue;
-        Frag f1[4][NB], f2[4][NB];
-        if (AHEAD) {
+            for (int n = 0; n < RB; ++n) {
+                const int id = threadIdx.x + n * 256, row = id / 16, kc = id % 16;
+                const long long off = src_off[row];
+                const int k = kb * 128 + kc * 8;
+                uint4 v = make_uint4(0, 0, 0, 0);
+                if (off >= 0 && k + 8 <= K) v = *reinterpret_cast<const uint4*>(src + off + k);
+                *reinterpret_cast<uint4*>(xt + row * XT_STRIDE + kc * 8) = v;
+            }
+            __syncthreads();
+            if (!active) continue;
+            Frag f1[4][NB], f2[4][NB];
 #pragma unroll
             for (int j = 0; j < 4; ++j)
 #pragma unroll
@@ -129,24 +130,73 @@ __device__ __forceinline__ void tile_product(const bf16_t* __restrict__ a1, cons
                     if (GATED) f2[j][i] = n2[j][i];
                 }
             fetch_a(min(kb + 1, kblocks - 1));           // (the last block once more rather than a branch around loads)
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int b = 0; b < RB; ++b) {
+                    Frag fx;
+                    fx.u = *reinterpret_cast<const uint4*>(xt + (b * 16 + r) * XT_STRIDE + c * 32 + j * 8);
+#pragma unroll
+                    for (int i = 0; i < NB; ++i) {
+                        acc1[i][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f1[j][i].v, fx.v, acc1[i][b], 0, 0, 0);
+                        if (GATED) acc2[i][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f2[j][i].v, fx.v, acc2[i][b], 0, 0, 0);
+                    }
+                }
         }
+        return;
+    }
+    // Large tiles: the rows of B of the block of k after the current one wait in registers while the current one is
+    // multiplied, and the fragments of A run one quarter block (32 columns of k) ahead of the products.
+    uint4 xr[RB];
+    auto fetch_x = [&](int kb) {
+#pragma unroll
+        for (int n = 0; n < RB; ++n) {
+            const int id = threadIdx.x + n * 256, row = id / 16, kc = id % 16;
+            const long long off = src_off[row];
+            const int k = kb * 128 + kc * 8;
+            xr[n] = make_uint4(0, 0, 0, 0);
+            if (off >= 0 && k + 8 <= K) xr[n] = *reinterpret_cast<const uint4*>(src + off + k);
+        }
+    };
+    Frag g1[NB], g2[NB];
+    auto fetch_quarter = [&](int q) {                    // quarter q of all: block q / 4, step q % 4 (the last one again past the end)
+        const int at = min(q, 4 * kblocks - 1);
+#pragma unroll
+        for (int i = 0; i < NB; ++i) {
+            g1[i] = frag_load(a1 + i * a_step + (size_t)(at / 4) * 2048 + (at % 4) * 512);
+            if (GATED) g2[i] = frag_load(a2 + i * a_step + (size_t)(at / 4) * 2048 + (at % 4) * 512);
+        }
+    };
+    __syncthreads();                                     // (src_off is written)
+    fetch_x(0);
+    if (active) fetch_quarter(0);
+    for (int kb = 0; kb < kblocks; ++kb) {
+        __syncthreads();
+#pragma unroll
+        for (int n = 0; n < RB; ++n) {
+            const int id = threadIdx.x + n * 256, row = id / 16, kc = id % 16;
+            *reinterpret_cast<uint4*>(xt + row * XT_STRIDE + kc * 8) = xr[n];
+        }
+        __syncthreads();
+        if (kb + 1 < kblocks) fetch_x(kb + 1);
+        if (!active) continue;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            if (!AHEAD) {
+            Frag f1[NB], f2[NB];
 #pragma unroll
-                for (int i = 0; i < NB; ++i) {
-                    f1[j][i] = frag_load(a1 + i * a_step + (size_t)kb * 2048 + j * 512);
-                    if (GATED) f2[j][i] = frag_load(a2 + i * a_step + (size_t)kb * 2048 + j * 512);
-                }
+            for (int i = 0; i < NB; ++i) {
+                f1[i] = g1[i];
+                if (GATED) f2[i] = g2[i];
             }
+            fetch_quarter(kb * 4 + j + 1);
 #pragma unroll
             for (int b = 0; b < RB; ++b) {
                 Frag fx;
                 fx.u = *reinterpret_cast<const uint4*>(xt + (b * 16 + r) * XT_STRIDE + c * 32 + j * 8);
 #pragma unroll
                 for (int i = 0; i < NB; ++i) {
-                    acc1[i][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f1[j][i].v, fx.v, acc1[i][b], 0, 0, 0);
-                    if (GATED) acc2[i][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f2[j][i].v, fx.v, acc2[i][b], 0, 0, 0);
+                    acc1[i][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f1[i].v, fx.v, acc1[i][b], 0, 0, 0);
+                    if (GATED) acc2[i][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f2[i].v, fx.v, acc2[i][b], 0, 0, 0);
                 }
             }
         }
@@ -156,7 +206,7 @@ __device__ __forceinline__ void tile_product(const bf16_t* __restrict__ a1, cons
 __device__ __forceinline__ float grouped_silu(float z) { return z / (1.0f + expf(-z)); }
 
 // gate and up products with the activation: hid[slot, f] (a tile has 16 RB slots)
-template <int RB>
+template <int RB, int NB>
 __global__ void __launch_bounds__(256) moe_gate_up_kernel(const bf16_t* __restrict__ x, const int* __restrict__ order,
                                                            const int* __restrict__ tile_expert,
                                                            const int* __restrict__ num_tiles,
@@ -185,7 +235,7 @@ __global__ void __launch_bounds__(256) moe_gate_up_kernel(const bf16_t* __restri
     for (int i = 0; i < NB; ++i)
 #pragma unroll
         for (int b = 0; b < RB; ++b) ag[i][b] = au[i][b] = (f32x4){0.f, 0.f, 0.f, 0.f};
-    tile_product<RB, true>(gate_t + block0, up_t + block0, a_step, x, src_off, D, active, xt, ag, au);
+    tile_product<RB, NB, true>(gate_t + block0, up_t + block0, a_step, x, src_off, D, active, xt, ag, au);
     if (!active) return;
     // the lane holds hidden units (nb + i) * 16 + 4 c .. + 4 of the slots 16 b + r
 #pragma unroll
@@ -204,7 +254,7 @@ __global__ void __launch_bounds__(256) moe_gate_up_kernel(const bf16_t* __restri
 }
 
 // down product: float32 rows in the order of the slots
-template <int RB>
+template <int RB, int NB>
 __global__ void __launch_bounds__(256) moe_down_grouped_kernel(const bf16_t* __restrict__ hid, const int* __restrict__ order,
                                                                 const int* __restrict__ tile_expert,
                                                                 const int* __restrict__ num_tiles,
@@ -231,7 +281,7 @@ __global__ void __launch_bounds__(256) moe_down_grouped_kernel(const bf16_t* __r
     for (int i = 0; i < NB; ++i)
 #pragma unroll
         for (int b = 0; b < RB; ++b) acc[i][b] = (f32x4){0.f, 0.f, 0.f, 0.f};
-    tile_product<RB, false>(wd, nullptr, a_step, hid, src_off, ff, active, xt, acc, unused);
+    tile_product<RB, NB, false>(wd, nullptr, a_step, hid, src_off, ff, active, xt, acc, unused);
     if (!active) return;
 #pragma unroll
     for (int i = 0; i < NB; ++i) {
@@ -291,16 +341,16 @@ extern "C" int tli_moe_grouped_bf16(const void* x, const int* ids, const float* 
     hipStream_t s = (hipStream_t)stream;
     hipLaunchKernelGGL(moe_sort_kernel, dim3(1), dim3(1024), 0, s, ids, (int)pairs, E, RT, (int)tiles_max, order, pos,
                        tile_expert, num_tiles);
-    const dim3 g1((ff + 64 * NB - 1) / (64 * NB), (unsigned)tiles_max), g2((D + 64 * NB - 1) / (64 * NB), (unsigned)tiles_max);
-#define TLI_GROUPED(RB)                                                                                              \
-    hipLaunchKernelGGL((moe_gate_up_kernel<RB>), g1, dim3(256), 0, s, (const bf16_t*)x, order, tile_expert, num_tiles, \
-                       (const bf16_t*)gate_t, (const bf16_t*)up_t, (bf16_t*)hid, top, D, ff);                        \
-    hipLaunchKernelGGL((moe_down_grouped_kernel<RB>), g2, dim3(256), 0, s, (const bf16_t*)hid, order, tile_expert,    \
-                       num_tiles, (const bf16_t*)down_t, part, D, ff)
-    if (RT == 16) { TLI_GROUPED(1); }
-    else if (RT == 32) { TLI_GROUPED(2); }
-    else if (RT == 64) { TLI_GROUPED(4); }
-    else { TLI_GROUPED(8); }
+#define TLI_GROUPED(RB, NBG)                                                                                          \
+    hipLaunchKernelGGL((moe_gate_up_kernel<RB, NBG>), dim3((ff + 64 * NBG - 1) / (64 * NBG), (unsigned)tiles_max),      \
+                       dim3(256), 0, s, (const bf16_t*)x, order, tile_expert, num_tiles, (const bf16_t*)gate_t,        \
+                       (const bf16_t*)up_t, (bf16_t*)hid, top, D, ff);                                                 \
+    hipLaunchKernelGGL((moe_down_grouped_kernel<RB, 2>), dim3((D + 127) / 128, (unsigned)tiles_max), dim3(256), 0, s,  \
+                       (const bf16_t*)hid, order, tile_expert, num_tiles, (const bf16_t*)down_t, part, D, ff)
+    if (RT == 16) { TLI_GROUPED(1, 2); }
+    else if (RT == 32) { TLI_GROUPED(2, 2); }
+    else if (RT == 64) { TLI_GROUPED(4, 2); }
+    else { TLI_GROUPED(8, 1); }
 #undef TLI_GROUPED
     hipLaunchKernelGGL(moe_combine_kernel, dim3(T), dim3(256), 0, s, part, pos, weights, (const bf16_t*)shared, shared_gate,
                        (bf16_t*)out, top, D);
