@@ -14,8 +14,8 @@
 // The matrices are read in the tiled layout of the other products (blocks of 16 rows x 128 columns, 4
 // KiB, in the order the operands of v_mfma_f32_16x16x32_bf16 want: a load instruction of a wave takes 1 KiB
 // in a row); rows and columns that do not exist are zeros there.  A is a tile of W (16 outputs), B the
-// rows of x, so a lane ends with 4 consecutive outputs of one row.  A wave takes 32 outputs and all RT
-// rows of its tile; the four waves of a workgroup share the rows of x through LDS.
+// rows of x, so a lane ends with 4 consecutive outputs of one row.  A wave takes 16 or 32 outputs and all
+// RT rows of its tile; the four waves of a workgroup share the rows of x through LDS.
 #include "common.h"
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
