@@ -55,6 +55,10 @@ SMALL = {
     # key head, a window longer than every test sequence, groups of one expert, a key size of 40, two taps
     "C": (_config(257, 100, [_layer("attention", _C_ATT, _C_MOE), _layer("delta", _delta(3, 1, 40, 20, 2), _C_MOE),
                              _layer("attention", _C_ATT, _C_MOE, 0)], emb_scale=2.0, eps=1e-6), 16, 11),
+    # whole heads of 64 turned (the attention kernels that norm, turn and write the cache themselves), four query heads
+    # on one key head, key heads of 128 on value heads of 32 in the delta rule, every group of experts kept
+    "F": (_config(300, 128, [_layer("delta", _delta(2, 1, 128, 32, 3), _moe(4, 2, 2, 2, 48, 64)),
+                             _layer("attention", _attention(4, 1, 64, 64, 40, 64), _moe(4, 2, 2, 2, 48, 64))], emb_scale=3.0), 16, 13),
     # heads of 64 (the matrix-core attention kernels), a delta state of 64 x 64, sixteen experts in four groups
     "R": (_config(320, 128, [_layer("attention", _attention(4, 2, 64, 64, 48, 32, base=50000.0), _moe(16, 4, 4, 2, 64, 128, scale=2.0)),
                              _layer("delta", _delta(4, 2, 64, 64, 4), _moe(16, 4, 4, 2, 64, 128, scale=2.0))]), 32, 7),
