@@ -22,25 +22,24 @@
 __device__ __forceinline__ float silu_f(float z) { return z / (1.0f + expf(-z)); }
 
 // ---------------------------------------------------------------------------------------------
-// prepare: one workgroup a row
+// prepare: a workgroup takes one row and one piece of it: a key head (its q and k vectors: convolution,
+// silu, unit vectors, their dot product; piece 0 also the row's beta and decay), or 256 channels of v
 // ---------------------------------------------------------------------------------------------
 template <typename T>
-__global__ void delta_prepare_kernel(const T* __restrict__ proj, int ld, const float* __restrict__ conv_w,
-                                     const T* __restrict__ kept, const float* __restrict__ ba, long long ba_row,
-                                     long long ba_col, const float* __restrict__ a_log, const float* __restrict__ dt_bias,
-                                     const int* __restrict__ positions, const int* __restrict__ seq_of_row,
-                                     const int* __restrict__ row_start, const int* __restrict__ slots,
-                                     float* __restrict__ qn, float* __restrict__ kn, float* __restrict__ vc,
-                                     float* __restrict__ beta, float* __restrict__ decay, float* __restrict__ qk,
-                                     int H, int G, int dk, int dv, int taps) {
-    extern __shared__ float buf[];                 // the row's channels after convolution and silu
-    const int r = blockIdx.x;
+__global__ void __launch_bounds__(256) delta_prepare_kernel(
+    const T* __restrict__ proj, int ld, const float* __restrict__ conv_w, const T* __restrict__ kept,
+    const float* __restrict__ ba, long long ba_row, long long ba_col, const float* __restrict__ a_log,
+    const float* __restrict__ dt_bias, const int* __restrict__ positions, const int* __restrict__ seq_of_row,
+    const int* __restrict__ row_start, const int* __restrict__ slots, float* __restrict__ qn, float* __restrict__ kn,
+    float* __restrict__ vc, float* __restrict__ beta, float* __restrict__ decay, float* __restrict__ qk, int H, int G,
+    int dk, int dv, int taps) {
+    __shared__ float scratch[16];
+    const int r = blockIdx.x, piece = blockIdx.y;
     const int seq = seq_of_row[r], pos = positions[r];
     const int in_step = r - row_start[seq];        // rows of this sequence that stand before r in the step
-    const int slot = slots[seq];
     const int qd = G * dk, C = 2 * qd + H * dv;
-    const T* mine = kept ? kept + (size_t)slot * (taps - 1) * C : nullptr;
-    for (int c = threadIdx.x; c < C; c += blockDim.x) {
+    const T* mine = kept ? kept + (size_t)slots[seq] * (taps - 1) * C : nullptr;
+    auto conv_silu = [&](int c) {
         float acc = 0.f;
         for (int j = 0; j < taps; ++j) {
             const int back = taps - 1 - j;          // the tap's row lies this many positions before r
@@ -50,40 +49,32 @@ __global__ void delta_prepare_kernel(const T* __restrict__ proj, int ld, const f
             else x = to_f32(mine[(size_t)(taps - 1 + in_step - back) * C + c]);
             acc = fmaf(conv_w[(size_t)j * C + c], x, acc);
         }
-        buf[c] = silu_f(acc);
+        return silu_f(acc);
+    };
+    if (piece >= G) {
+        const int c = (piece - G) * 256 + threadIdx.x;
+        if (c < H * dv) vc[(size_t)r * H * dv + c] = conv_silu(2 * qd + c);
+        return;
     }
-    __syncthreads();
-    const int lane = threadIdx.x % TLI_WAVE, wave = threadIdx.x / TLI_WAVE, waves = blockDim.x / TLI_WAVE;
-    // unit vectors: the 2 G heads of q and k, a wave each in turn
-    for (int v = wave; v < 2 * G; v += waves) {
-        float* x = buf + (size_t)v * dk;
-        float ss = 0.f;
-        for (int i = lane; i < dk; i += TLI_WAVE) ss += x[i] * x[i];
-        ss = wave_sum(ss);
-        float scale = 1.0f / sqrtf(ss + 1e-6f);
-        if (v < G) scale *= 1.0f / sqrtf((float)dk);
-        float* out = (v < G ? qn : kn) + (size_t)r * qd + (size_t)(v < G ? v : v - G) * dk;
-        for (int i = lane; i < dk; i += TLI_WAVE) {
-            const float y = x[i] * scale;
-            x[i] = y;
-            out[i] = y;
-        }
+    const int i = threadIdx.x;                      // dk <= 256: an element of q and of k a thread
+    const bool has = i < dk;
+    const float q = has ? conv_silu(piece * dk + i) : 0.f;
+    const float k = has ? conv_silu(qd + piece * dk + i) : 0.f;
+    const float sq = block_sum(q * q, scratch), sk = block_sum(k * k, scratch);
+    const float qu = q * (1.0f / sqrtf(sq + 1e-6f)) * (1.0f / sqrtf((float)dk));
+    const float ku = k * (1.0f / sqrtf(sk + 1e-6f));
+    const float dot = block_sum(qu * ku, scratch);
+    if (has) {
+        qn[(size_t)r * qd + (size_t)piece * dk + i] = qu;
+        kn[(size_t)r * qd + (size_t)piece * dk + i] = ku;
     }
-    for (int i = threadIdx.x; i < H * dv; i += blockDim.x) vc[(size_t)r * H * dv + i] = buf[2 * qd + i];
-    if (threadIdx.x < H) {
-        const int h = threadIdx.x;
-        const float b = ba[(size_t)r * ba_row + (size_t)h * ba_col];
-        const float a = ba[(size_t)r * ba_row + (size_t)(H + h) * ba_col] + dt_bias[h];
-        beta[(size_t)r * H + h] = 1.0f / (1.0f + expf(-b));
+    if (i == 0) qk[(size_t)r * G + piece] = dot;
+    if (piece == 0 && i < H) {
+        const float b = ba[(size_t)r * ba_row + (size_t)i * ba_col];
+        const float a = ba[(size_t)r * ba_row + (size_t)(H + i) * ba_col] + dt_bias[i];
+        beta[(size_t)r * H + i] = 1.0f / (1.0f + expf(-b));
         const float sp = fmaxf(a, 0.f) + log1pf(expf(-fabsf(a)));
-        decay[(size_t)r * H + h] = expf(-expf(a_log[h]) * sp);
-    }
-    __syncthreads();
-    for (int g = wave; g < G; g += waves) {
-        float d = 0.f;
-        for (int i = lane; i < dk; i += TLI_WAVE) d = fmaf(buf[(size_t)g * dk + i], buf[(size_t)(G + g) * dk + i], d);
-        d = wave_sum(d);
-        if (lane == 0) qk[(size_t)r * G + g] = d;
+        decay[(size_t)r * H + i] = expf(-expf(a_log[i]) * sp);
     }
 }
 
@@ -273,18 +264,19 @@ extern "C" int tli_delta_prepare(const void* proj, int ld, const float* conv_w, 
     if (ld < C) return tli_fail("delta_prepare: rows of %d hold fewer than the %d channels", ld, C);
     if (taps > 1 && !kept) return tli_fail("delta_prepare: %d taps need the sequences' kept rows", taps);
     if (H > 256) return tli_fail("delta_prepare: at most 256 heads, got %d", H);
-    const size_t lds = (size_t)C * sizeof(float);
-    if (lds > 64 * 1024) return tli_fail("delta_prepare: %d channels do not fit the workgroup's memory", C);
+    if (dk > DELTA_MAX_DK) return tli_fail("delta_prepare: key heads of at most %d, got %d", DELTA_MAX_DK, dk);
+    if (G + (H * dv + 255) / 256 > 65535) return tli_fail("delta_prepare: too many channels for one launch");
+    const dim3 grid(T, G + (H * dv + 255) / 256);
     hipStream_t s = (hipStream_t)stream;
     if (dtype == TLI_F32) {
-        hipLaunchKernelGGL((delta_prepare_kernel<float>), dim3(T), dim3(256), lds, s, (const float*)proj, ld, conv_w,
+        hipLaunchKernelGGL((delta_prepare_kernel<float>), grid, dim3(256), 0, s, (const float*)proj, ld, conv_w,
                            (const float*)kept, ba, ba_row, ba_col, a_log, dt_bias, positions, seq_of_row, row_start, slots, qn, kn, vc,
                            beta, decay, qk, H, G, dk, dv, taps);
         if (taps > 1)
             hipLaunchKernelGGL((delta_conv_keep_kernel<float>), dim3((C + 255) / 256, seqs), dim3(256), 0, s,
                                (const float*)proj, ld, (float*)kept, row_start, seq_start, slots, C, taps);
     } else if (dtype == TLI_BF16) {
-        hipLaunchKernelGGL((delta_prepare_kernel<bf16_t>), dim3(T), dim3(256), lds, s, (const bf16_t*)proj, ld, conv_w,
+        hipLaunchKernelGGL((delta_prepare_kernel<bf16_t>), grid, dim3(256), 0, s, (const bf16_t*)proj, ld, conv_w,
                            (const bf16_t*)kept, ba, ba_row, ba_col, a_log, dt_bias, positions, seq_of_row, row_start, slots, qn, kn,
                            vc, beta, decay, qk, H, G, dk, dv, taps);
         if (taps > 1)

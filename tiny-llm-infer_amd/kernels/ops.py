@@ -1079,8 +1079,6 @@ class HipOps:
             raise KernelError(f"a state of {dk} x {dv} a head is not supported: key heads of 1 to {self.MAX_DELTA_KEY_DIM}")
         if not 1 <= taps <= self.MAX_CONV_TAPS:
             raise KernelError(f"a convolution of {taps} taps is not supported: 1 to {self.MAX_CONV_TAPS}")
-        if (2 * kv_heads * dk + heads * dv) * 4 > 64 * 1024:
-            raise KernelError("the channels of q, k and v of a row do not fit a workgroup's memory")
 
     def small_product(self, x: torch.Tensor, w_rows: torch.Tensor):
         """x W^T in float32 for a matrix of few rows (a router, a few numbers a head): returns (y, transposed).
