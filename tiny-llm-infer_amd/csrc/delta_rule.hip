@@ -187,23 +187,17 @@ __global__ __launch_bounds__(256) void delta_recurrence_kernel(
         __syncthreads();
         if (c0 + CT < r1) fetch(c0 + CT);
         const int rows = min(CT, r1 - c0);
-        // the row after the current one is read from LDS while the current one is worked on
-        float kx[RPT], qx[RPT], vx, bx, gx, cx;
-        auto read_row = [&](int t) {
+        // the row after the current one is read from LDS while the current one is worked on: two sets of
+        // registers take turns, two rows a round of the loop
+        auto read_row = [&](int t, float (&kx)[RPT], float (&qx)[RPT], float (&sx)[4]) {
             const float* kp = ks + t * DKP + part * RPT;
             const float* qp = qs + t * DKP + part * RPT;
 #pragma unroll
             for (int r = 0; r < RPT; ++r) { kx[r] = kp[r]; qx[r] = qp[r]; }
-            vx = vs[t * DELTA_COLS + local];
-            bx = sc[t]; gx = sc[CT + t]; cx = sc[2 * CT + t];
+            sx[0] = vs[t * DELTA_COLS + local];
+            sx[1] = sc[t]; sx[2] = sc[CT + t]; sx[3] = sc[2 * CT + t];
         };
-        read_row(0);
-        for (int t = 0; t < rows; ++t) {
-            float k[RPT], q[RPT];
-#pragma unroll
-            for (int r = 0; r < RPT; ++r) { k[r] = kx[r]; q[r] = qx[r]; }
-            const float v0 = vx, b0 = bx, g0 = gx, c0q = cx;
-            read_row(min(t + 1, CT - 1));
+        auto walk_row = [&](int t, const float (&k)[RPT], const float (&q)[RPT], const float (&sx)[4]) {
             float d1[2] = {0.f, 0.f}, d2[2] = {0.f, 0.f};          // two sums each: shorter chains of dependent additions
 #pragma unroll
             for (int r = 0; r < RPT; ++r) {
@@ -211,11 +205,22 @@ __global__ __launch_bounds__(256) void delta_recurrence_kernel(
                 d2[r & 1] = fmaf(q[r], S[r], d2[r & 1]);
             }
             const float s1 = row16_sum(d1[0] + d1[1]), s2 = row16_sum(d2[0] + d2[1]);
-            const float u = b0 * (v0 - g0 * s1);
+            const float g0 = sx[2];
+            const float u = sx[1] * (sx[0] - g0 * s1);
 #pragma unroll
             for (int r = 0; r < RPT; ++r) S[r] = fmaf(k[r], u, g0 * S[r]);
-            if (part == 0 && live) out[(size_t)(c0 + t) * vd + (size_t)head * dv + col] = fmaf(c0q, u, g0 * s2);
+            if (part == 0 && live) out[(size_t)(c0 + t) * vd + (size_t)head * dv + col] = fmaf(sx[3], u, g0 * s2);
+        };
+        float ka[RPT], qa[RPT], sa[4], kb[RPT], qb[RPT], sb[4];
+        read_row(0, ka, qa, sa);
+        int t = 0;
+        for (; t + 1 < rows; t += 2) {
+            read_row(t + 1, kb, qb, sb);
+            walk_row(t, ka, qa, sa);
+            read_row(min(t + 2, CT - 1), ka, qa, sa);
+            walk_row(t + 1, kb, qb, sb);
         }
+        if (t < rows) walk_row(t, ka, qa, sa);
     }
 #pragma unroll
     for (int r = 0; r < RPT; ++r) mine[(size_t)r * DELTA_COLS * DELTA_LANES] = S[r];
