@@ -107,41 +107,49 @@ __device__ __forceinline__ void tile_product(const bf16_t* __restrict__ a1, cons
             }
     };
     if (AHEAD) {
-        if (active) fetch_a(0);
-        for (int kb = 0; kb < kblocks; ++kb) {
-            __syncthreads();
+        // no LDS and no barrier in the loop: a wave reads its fragments of the few rows of B itself (the four waves
+        // of the workgroup read the same ones, from the cache), a block ahead like those of A
+        __syncthreads();                                 // (src_off is written)
+        if (!active) return;
+        long long off[RB];
 #pragma unroll
-            for (int n = 0; n < RB; ++n) {
-                const int id = threadIdx.x + n * 256, row = id / 16, kc = id % 16;
-                const long long off = src_off[row];
-                const int k = kb * 128 + kc * 8;
-                uint4 v = make_uint4(0, 0, 0, 0);
-                if (off >= 0 && k + 8 <= K) v = *reinterpret_cast<const uint4*>(src + off + k);
-                *reinterpret_cast<uint4*>(xt + row * XT_STRIDE + kc * 8) = v;
-            }
-            __syncthreads();
-            if (!active) continue;
-            Frag f1[4][NB], f2[4][NB];
+        for (int b = 0; b < RB; ++b) off[b] = src_off[b * 16 + r];
+        Frag xn[4][RB];
+        auto fetch_b = [&](int kb) {
 #pragma unroll
             for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int b = 0; b < RB; ++b) {
+                    const int k = kb * 128 + c * 32 + j * 8;
+                    xn[j][b].u = make_uint4(0, 0, 0, 0);
+                    if (off[b] >= 0 && k + 8 <= K) xn[j][b].u = *reinterpret_cast<const uint4*>(src + off[b] + k);
+                }
+        };
+        fetch_a(0);
+        fetch_b(0);
+        for (int kb = 0; kb < kblocks; ++kb) {
+            Frag f1[4][NB], f2[4][NB], fx[4][RB];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
 #pragma unroll
                 for (int i = 0; i < NB; ++i) {
                     f1[j][i] = n1[j][i];
                     if (GATED) f2[j][i] = n2[j][i];
                 }
+#pragma unroll
+                for (int b = 0; b < RB; ++b) fx[j][b] = xn[j][b];
+            }
             fetch_a(min(kb + 1, kblocks - 1));           // (the last block once more rather than a branch around loads)
+            fetch_b(min(kb + 1, kblocks - 1));
 #pragma unroll
             for (int j = 0; j < 4; ++j)
 #pragma unroll
-                for (int b = 0; b < RB; ++b) {
-                    Frag fx;
-                    fx.u = *reinterpret_cast<const uint4*>(xt + (b * 16 + r) * XT_STRIDE + c * 32 + j * 8);
+                for (int b = 0; b < RB; ++b)
 #pragma unroll
                     for (int i = 0; i < NB; ++i) {
-                        acc1[i][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f1[j][i].v, fx.v, acc1[i][b], 0, 0, 0);
-                        if (GATED) acc2[i][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f2[j][i].v, fx.v, acc2[i][b], 0, 0, 0);
+                        acc1[i][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f1[j][i].v, fx[j][b].v, acc1[i][b], 0, 0, 0);
+                        if (GATED) acc2[i][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f2[j][i].v, fx[j][b].v, acc2[i][b], 0, 0, 0);
                     }
-                }
         }
         return;
     }
